@@ -566,8 +566,7 @@ __global__ __launch_bounds__(NT, 1) void gemm256_kernel(Args a) {
           constexpr int q = 4 * (g % GPS) + qq;
           // the previous call's F0 reads (order 2) are waited for here, per A fragment: row 0 (A0,
           // all B) before MFMA 0 (A1.. and this call's first read may still be in flight), row 1 (A1)
-          // before MFMA 8; rows 2.. are covered by barrier #1's lgkmcnt(0).  No copy of a fragment
-          // register sits between (checked in the disassembly: the loop has no v_mov)
+          // before MFMA 8; rows 2.. are covered by barrier #1's lgkmcnt(0).
           if constexpr (g < 4 && q == 0) wait_lgkm<TN>();
           if constexpr (g < 4 && q == 8) wait_lgkm<TN + 7>();
           if constexpr (g < GPS) mfma_acc(acc[q >> 3][q & 7], fa0[q >> 3], fb0[q & 7]);

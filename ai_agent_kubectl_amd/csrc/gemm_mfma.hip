@@ -275,8 +275,7 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(Args a) {
   // every kernel argument the k-loop needs is read into registers here, before the loop: under
   // KA_GM_PIPE 2 the asm fragment reads are waited for with a counted lgkmcnt, which a scalar
   // (s_load) kernarg read issued between the reads and that wait would break.  The asm makes wnt an
-  // opaque SGPR value, so hipcc cannot rematerialise it from the kernarg segment inside the loop
-  // (build.py check_lgkm_windows verifies the k-loop's read windows in the generated assembly).
+  // opaque SGPR value, so hipcc cannot rematerialise it from the kernarg segment inside the loop.
   int wnt = a.wnt;
   asm volatile("" : "+s"(wnt));
   // the wave's pieces of a stage, W pieces then X pieces; part 0 / 1: the first / second half of that

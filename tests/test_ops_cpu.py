@@ -95,29 +95,6 @@ def test_plan_for_takes_the_next_bucket_up():
         ops.GEMM_PLAN.update(saved)
 
 
-def test_lgkm_window_checker_flags_compiler_lgkm_ops():
-    """build.py re-verifies that no compiler-issued LGKM operation sits between the
-    k-loop's asm fragment reads and their counted lgkmcnt wait (gemm_mfma KA_GM_PIPE 2, gemm_big)."""
-    from ai_agent_kubectl_amd.build import lgkm_window_violations
-    ok = """_ZN2gm11gemm_kernelI1EEvNS_4ArgsE:
-\t;;#ASMSTART
-\tds_read_b128 v[0:3], v10 offset:0
-\t;;#ASMEND
-\tv_mfma_f32_16x16x32_bf16 a[0:3], v[4:7], v[8:11], a[0:3]
-\t;;#ASMSTART
-\ts_waitcnt lgkmcnt(4)
-\t;;#ASMEND
-\ts_load_dword s4, s[0:1], 0x10
-\tds_write_b32 v1, v2
-"""
-    n, bad = lgkm_window_violations(ok, "gemm_kernel")
-    assert n == 1 and bad == []
-    broken = ok.replace("\tv_mfma", "\ts_load_dwordx2 s[6:7], s[0:1], 0x8\n\tv_mfma")
-    n, bad = lgkm_window_violations(broken, "gemm_kernel")
-    assert n == 1 and len(bad) == 1 and "s_load_dwordx2" in bad[0][2]
-    assert lgkm_window_violations(broken, "other_kernel") == (0, [])
-
-
 def test_plan_ladder_anomalies_flags_slower_smaller_bucket():
     """a bucket whose planned GEMM time exceeds the next larger bucket's (whose
     plan also runs the smaller M) is a tuning miss; ladder_anomalies finds it per (N, K, consumer)."""
@@ -143,27 +120,6 @@ def test_repair_ladder_takes_the_larger_buckets_plan():
     assert plans["32,32000,4096,plain"][:4] == ["gm", 1, 5, 40.0] and plans["32,32000,4096,plain"][4] == 52.6
     assert plans["2,4096,4096,norm"][0] == "rows" and plans["1,4096,4096,norm"][:3] == ["rows", 1, 2]
     assert [a[0] for a in ladder_anomalies(plans)] == ["16,4096,4096,norm"]   # blas above: left alone
-
-
-def test_mfma_span_valu_checker():
-    """build.py refuses a gemm_big build whose all-asm k-loop got a compiler VALU instruction between
-    asm MFMAs (a WAR hazard on operands hipcc cannot see being read)."""
-    from ai_agent_kubectl_amd.build import mfma_span_valu
-    ok = """_ZN2gb14gemm256_kernelILi3ELi8EEEvNS_4ArgsE:
-\tv_mov_b32 v1, 0
-\t;;#ASMSTART
-\tv_mfma_f32_16x16x32_bf16 a[0:3], v[56:59], v[4:7], a[0:3]
-\t;;#ASMEND
-\ts_and_b64 vcc, exec, s[4:5]
-\t;;#ASMSTART
-\tv_mfma_f32_16x16x32_bf16 a[4:7], v[56:59], v[8:11], a[4:7]
-\t;;#ASMEND
-\tv_add_u32 v2, v1, v3
-"""
-    assert mfma_span_valu(ok, "gemm256_kernel") == []
-    bad = ok.replace("\ts_and_b64", "\tv_cndmask_b32_e64 v56, 0, 1, s[58:59]\n\ts_and_b64")
-    got = mfma_span_valu(bad, "gemm256_kernel")
-    assert len(got) == 1 and "v_cndmask" in got[0][2]
 
 
 def test_prefill_gemm_plan_buckets():
