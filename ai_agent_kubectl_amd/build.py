@@ -3,6 +3,9 @@
 * `build_hip()`    — compiles every `csrc/*.hip` for gfx950 with hipcc into
                      `ops/lib/libkagent_hip.so` (one object per source, compiled in parallel,
                      then linked).  Cross-compiles without a GPU.
+* `build_mixers()` — only the sources tagged `// KA_HIP_LIB: mixers` (the kernels of the models with an
+                     fp32 residual stream) into `ops/lib/libkagent_mixers.so`: a few seconds, so a
+                     fresh checkout that serves only such a model builds just this.
 * `build_runtime()`— compiles the C++ host runtime (`runtime/*.cpp`: tokenizer trie, paged-KV
                      block manager, batch-metadata builder) into `runtime/_native*.so` via pybind11.
 
@@ -21,6 +24,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 LIB_DIR = os.path.join(PKG, "ops", "lib")
 HIP_LIB = os.path.join(LIB_DIR, "libkagent_hip.so")
+MIXERS_LIB = os.path.join(LIB_DIR, "libkagent_mixers.so")
 RUNTIME_DIR = os.path.join(PKG, "runtime")
 ARCH = os.environ.get("KA_OFFLOAD_ARCH", "gfx950")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -51,16 +55,32 @@ def file_flags(src: str):
     return []
 
 
-def build_hip(force: bool = False, verbose: bool = False, extra_flags=(), out: str = "") -> str:
+def lib_tag(src: str) -> str:
+    """The library a source belongs to: its `// KA_HIP_LIB: <name>` header line, or "" (the main one)."""
+    with open(src) as f:
+        for i, line in enumerate(f):
+            if line.startswith("// KA_HIP_LIB:"):
+                return line.split(":", 1)[1].strip()
+            if i > 40:
+                break
+    return ""
+
+
+def build_mixers(force: bool = False, verbose: bool = False) -> str:
+    return build_hip(force, verbose, out=MIXERS_LIB, tag="mixers")
+
+
+def build_hip(force: bool = False, verbose: bool = False, extra_flags=(), out: str = "", tag: str = "") -> str:
     """out: another library path (an A/B build with `extra_flags`, e.g. -DKA_GM_SCHED=0, loaded only by
-    diagnostic runs: ops/_hip.py KA_HIP_LIB + KA_HIP_LIB_DIAG=1); its objects go next to it."""
-    srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    diagnostic runs: ops/_hip.py KA_HIP_LIB + KA_HIP_LIB_DIAG=1); its objects go next to it.
+    tag: the sources of that `KA_HIP_LIB` tag only ("" = the untagged ones, the main library)."""
+    srcs = sorted(s for s in glob.glob(os.path.join(CSRC, "*.hip")) if lib_tag(s) == tag)
     headers = glob.glob(os.path.join(CSRC, "*.h"))
     lib = out or HIP_LIB
     os.makedirs(os.path.dirname(lib), exist_ok=True)
     if not force and not _newer(srcs + headers, lib):
         return lib
-    obj_dir = os.path.join(os.path.dirname(lib), "obj") if out else os.path.join(LIB_DIR, "obj")
+    obj_dir = os.path.join(os.path.dirname(lib), "obj") if out and not tag else os.path.join(LIB_DIR, "obj")
     os.makedirs(obj_dir, exist_ok=True)
     flags = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-munsafe-fp-atomics",
              "-Wno-unused-result", *extra_flags]
@@ -105,7 +125,7 @@ def build_runtime(force: bool = False, verbose: bool = False) -> str:
 
 
 def build_all(force: bool = False, verbose: bool = True):
-    return build_hip(force, verbose), build_runtime(force, verbose)
+    return build_hip(force, verbose), build_mixers(force, verbose), build_runtime(force, verbose)
 
 
 if __name__ == "__main__":

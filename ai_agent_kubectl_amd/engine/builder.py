@@ -7,6 +7,7 @@ workload.
 """
 from __future__ import annotations
 
+import glob
 import logging
 import os
 import time
@@ -44,6 +45,7 @@ class EngineOptions:
     safe_decode: bool = True
     ignore_eos: bool = False
     prefix_caching: bool = True
+    dtype: str = "bfloat16"         # "float32": weights, activations and cache in fp32 (families that support it)
 
     @classmethod
     def from_settings(cls, s) -> "EngineOptions":
@@ -66,7 +68,18 @@ def build_engine(opts: EngineOptions, comm=None, metrics=None) -> LLMEngine:
         from ..ops._hip import require
         require()  # fail loudly: the GPU path never runs without the HIP kernels
         torch.cuda.set_device(dev.index if dev.index is not None else torch.cuda.current_device())
-    dtype = torch.bfloat16
+    if opts.dtype not in ("bfloat16", "float32"):
+        raise ValueError(f"dtype {opts.dtype!r}: bfloat16 or float32")
+    dtype = torch.float32 if opts.dtype == "float32" else torch.bfloat16
+    family = getattr(cfg, "family", "llama")
+    if dtype == torch.float32 and family in ("llama", "mixtral"):
+        raise ValueError("the Llama / Mixtral kernels are bf16; float32 is served by the fp32-residual families (vivepel)")
+    if dtype == torch.float32:   # true fp32 products: no reduced-precision matrix mode
+        torch.backends.cuda.matmul.allow_tf32 = False
+        torch.backends.cudnn.allow_tf32 = False
+    weights_spec = opts.weights
+    if os.path.isdir(opts.model) and weights_spec.startswith("random") and glob.glob(os.path.join(opts.model, "*.safetensors")):
+        weights_spec = opts.model   # MODEL names a checkpoint folder: its config.json and its tensors
     # MoE: experts are sharded over the tensor-parallel group (EP = TP); the all-reduce after the
     # MoE block is the expert combine.  EP is therefore derived, not free (EP=1 with TP>1 would
     # replicate experts and double-count them in that all-reduce).
@@ -74,9 +87,12 @@ def build_engine(opts: EngineOptions, comm=None, metrics=None) -> LLMEngine:
     if cfg.is_moe and opts.ep_size not in (1, opts.tp_size):
         raise ValueError("EP must equal TP (experts are sharded over the tensor-parallel group)")
     par = ParallelInfo(opts.tp_rank, opts.tp_size, opts.tp_rank if ep_size > 1 else 0, ep_size)
-    weights = build_weights(opts.weights, cfg, par, device=dev, dtype=dtype)
+    weights = build_weights(weights_spec, cfg, par, device=dev, dtype=dtype)
     # ---- KV pool size ----
-    per_block = cfg.num_layers * 2 * (cfg.num_kv_heads // opts.tp_size) * cfg.head_dim * opts.block_size * 2
+    if family in ("llama", "mixtral"):
+        per_block = cfg.num_layers * 2 * (cfg.num_kv_heads // opts.tp_size) * cfg.head_dim * opts.block_size * 2
+    else:
+        per_block = cfg.kv_bytes_per_token(4 if dtype == torch.float32 else 2) * opts.block_size
     # KV_CACHE_TOKENS of pooled KV (not max_batch x max_model_len: with an 8192-token context that
     # would be 2M tokens); at least one full-length sequence fits, the rest is preemption's job.
     # The serving default (KV_CACHE_TOKENS unset / 0) takes the whole GPU_MEM_FRACTION budget left
@@ -99,6 +115,9 @@ def build_engine(opts: EngineOptions, comm=None, metrics=None) -> LLMEngine:
     else:
         want = opts.kv_cache_tokens // opts.block_size if opts.kv_cache_tokens > 0 else 4096
         num_blocks = min(max(want, min_blocks), 4096)
+    if dev.type == "cuda" and family == "vivepel":
+        from ..ops._hip import require_mixers
+        require_mixers()
     masks = build_masks(tok, allow_eos=not opts.ignore_eos) if opts.safe_decode else None
     if comm is not None and opts.tp_size > 1:
         from ..parallel.custom_allreduce import maybe_enable

@@ -24,7 +24,8 @@ import torch
 
 from ..models.config import ModelConfig
 from .. import ops
-from ..models.llama import AttnMeta, LlamaModel
+from ..models import model_class
+from ..models.llama import AttnMeta
 
 logger = logging.getLogger("app.engine")
 from ..parallel.comm import LocalComm
@@ -84,16 +85,14 @@ class ModelRunner:
         # engine schedules the step after it once that event has passed (engine._lookahead_step)
         self.lookahead_layers = int(os.environ.get("KA_LOOKAHEAD_LAYERS", "10"))
         self.tp_rank, self.tp_size = tp_rank, tp_size
-        self.model = LlamaModel(cfg, weights, self.comm, tp_rank, tp_size, ep_rank, ep_size)
+        # the model class of the configuration's family (models/__init__.py); the model owns the
+        # layout of its paged cache (one tensor over all layers for Llama, one per layer where
+        # the layers differ), the runner and the block manager only deal in pages
+        self.model = model_class(cfg)(cfg, weights, self.comm, tp_rank, tp_size, ep_rank, ep_size)
         self.block_size = block_size
         self.num_blocks = num_blocks
         self.max_blocks = (max_model_len + block_size - 1) // block_size
-        hkv = cfg.num_kv_heads // tp_size
-        L, D = cfg.num_layers, cfg.head_dim
-        dt = weights["embed"].dtype
-        # zero-filled: stale slots read by masked lanes must be finite (attention.hip contract)
-        self.k_cache = torch.zeros((L, num_blocks, hkv, block_size, D), dtype=dt, device=self.device)
-        self.v_cache = torch.zeros((L, num_blocks, hkv, D, block_size), dtype=dt, device=self.device)
+        self.k_cache, self.v_cache = self.model.alloc_cache(num_blocks, block_size)
         self.mask_bits = (torch.from_numpy(mask_bits.view(np.int32)).to(self.device)
                           if mask_bits is not None else None)
         self.buckets = sorted(set(int(b) for b in graph_buckets))
@@ -166,18 +165,22 @@ class ModelRunner:
         return self.cascade_min_b > 0 and B >= self.cascade_min_b and self.device.type == "cuda"
 
     def _decode_forward(self, B: int) -> None:
-        meta = AttnMeta(positions=self._view("pos", B), slot_mapping=self._view("slots", B),
-                        block_tables=self._view("bt", B), ctx_lens=self._view("ctx", B),
-                        logits_indices=self.d_logits_idx[:B], is_decode=True,
-                        shared_blocks=self._view("nsh", 1) if self._cascade(B) else None)
-        h = self.model.forward(self._view("ids", B), meta, self.k_cache, self.v_cache)
+        h = self._decode_hidden(B)
         mask_idx = self._view("mask", B) if self.mask_bits is not None else None
         tok = self.model.sample(h, self.mask_bits, mask_idx)
         self.d_out[:B].copy_(tok)
 
+    def _decode_hidden(self, B: int) -> torch.Tensor:
+        """The model's forward over the decode staging image: final-normed hidden states [B, H]."""
+        meta = AttnMeta(positions=self._view("pos", B), slot_mapping=self._view("slots", B),
+                        block_tables=self._view("bt", B), ctx_lens=self._view("ctx", B),
+                        logits_indices=self.d_logits_idx[:B], is_decode=True,
+                        shared_blocks=self._view("nsh", 1) if self._cascade(B) else None)
+        return self.model.forward(self._view("ids", B), meta, self.k_cache, self.v_cache)
+
     def autotune(self) -> dict:
         """Pick hipBLASLt vs the hand-written decode GEMM per (bucket, N, K) on this model's weights."""
-        if self.device.type != "cuda":
+        if self.device.type != "cuda" or not self._llama_kernels():
             return {}
         from ..ops.autotune import tune_linear
         groups = {}
@@ -228,7 +231,7 @@ class ModelRunner:
         fills ops.LM_HEAD_FUSED and the threshold for untimed row counts."""
         m = self.model
         lm = m.W["lm_head"]
-        if self.device.type != "cuda" or ops.LM_HEAD_MODE != "auto":
+        if self.device.type != "cuda" or ops.LM_HEAD_MODE != "auto" or not self._llama_kernels():
             return {}
         from ..ops.autotune import _time, load_section, plan_mode, save_section
         K = lm.shape[1]
@@ -274,7 +277,7 @@ class ModelRunner:
         KA_PREFILL_MARGIN (default 0.02) of hipBLASLt."""
         m = self.model
         ops.PREFILL_PLAN.clear()
-        if self.device.type != "cuda" or ops.PREFILL_GEMM != "auto":
+        if self.device.type != "cuda" or ops.PREFILL_GEMM != "auto" or not self._llama_kernels():
             return {}
         from ..ops.autotune import _time, load_section, plan_mode, save_section
         margin = float(os.environ.get("KA_PREFILL_MARGIN", "0.02"))
@@ -315,7 +318,8 @@ class ModelRunner:
         rotated over layers; fills ops.DECODE_SWIGLU_CFG with the winners."""
         m = self.model
         ops.DECODE_SWIGLU_CFG.clear()
-        if self.device.type != "cuda" or ops.DECODE_SWIGLU == "0" or getattr(m.cfg, "is_moe", False):
+        if (self.device.type != "cuda" or ops.DECODE_SWIGLU == "0" or getattr(m.cfg, "is_moe", False)
+                or not self._llama_kernels()):
             return {}
         ws = [L["w13"] for L in m.layers if L.get("w13") is not None and L["w13"].dim() == 2][:8]
         if not ws:
@@ -369,6 +373,11 @@ class ModelRunner:
         logger.info("decode swiglu plan: %s", report)
         return report
 
+    def _llama_kernels(self) -> bool:
+        """The model runs the Llama kernel set (hand-written GEMM plans, fused LM head, gemm_big workspace):
+        the tuning passes apply.  Other families bring their own ops and vendor GEMMs."""
+        return getattr(self.cfg, "family", "llama") in ("llama", "mixtral")
+
     def _attention_consumer(self, ctx: int = 128):
         """fn(qkv, M): decode_attention_rope over M synthetic sequences of `ctx` cached tokens in
         layer 0's cache (autotune runs before serving: the KV written here is never read)."""
@@ -394,7 +403,7 @@ class ModelRunner:
         if not self.use_graphs:
             return 0.0
         t0 = time.perf_counter()
-        if self.device.type == "cuda":
+        if self.device.type == "cuda" and self._llama_kernels():
             ops.gemm_big_ws(self.device)   # allocated (and zeroed) outside any capture
         if autotune:
             self.gemm_plan = self.autotune()
@@ -745,6 +754,13 @@ class ModelRunner:
     def _run_prefill(self, buf: torch.Tensor, T: int, S: int, max_q: int, nc: int = 0, nd: int = 0,
                      t_real: int = 0) -> torch.Tensor:
         mb = self.max_blocks
+        ids, meta, mask = self._prefill_meta(buf, T, S, max_q, nc, nd, t_real)
+        h = self.model.forward(ids, meta, self.k_cache, self.v_cache)
+        return self.model.sample(h, self.mask_bits, mask if self.mask_bits is not None else None)
+
+    def _prefill_meta(self, buf: torch.Tensor, T: int, S: int, max_q: int, nc: int = 0, nd: int = 0, t_real: int = 0):
+        """Unpack `_pack_prefill`'s image on the device (after the step's KV block copies): ids, AttnMeta, mask rows."""
+        mb = self.max_blocks
         if nc:
             n = buf.shape[0]
             ops.kv_block_copy(self.k_cache, self.v_cache, buf[n - 2 * nc:n - nc], buf[n - nc:])
@@ -758,8 +774,53 @@ class ModelRunner:
         meta = AttnMeta(positions=pos, slot_mapping=slots, block_tables=bt, ctx_lens=ctx, logits_indices=lidx,
                         is_decode=False, q_starts=q_starts, max_q_len=max_q, num_decode=nd,
                         num_tokens=t_real or T)
-        h = self.model.forward(ids, meta, self.k_cache, self.v_cache)
-        return self.model.sample(h, self.mask_bits, mask if self.mask_bits is not None else None)
+        return ids, meta, mask
+
+    @torch.inference_mode()
+    def execute_logits(self, batch: Batch, rows: List[List[int]]) -> torch.Tensor:
+        """One step for `batch` through the same packing, cache and forward as `execute`, but instead of
+        sampling it returns logits: fp32 [sum(len(r) for r in rows), vocab], for rows[i] = offsets among
+        sequence i's tokens of this step, in batch order.  (TP = 1; trace replay, logit-level tests.)"""
+        assert self.tp_size == 1 and len(rows) == len(batch.seqs)
+        B = len(batch.seqs)
+        if B == 0:
+            return torch.empty((0, self.cfg.vocab_size), dtype=torch.float32, device=self.device)
+        if batch.is_decode and B <= self.bmax:
+            i = bisect.bisect_left(self.buckets, B)
+            Bp = self.buckets[i] if i < len(self.buckets) else B
+            self._pack_decode(batch, Bp)
+            n_copy = self._off["bt"] + Bp * self.max_blocks
+            self.d_stage[:n_copy].copy_(self.h_stage[:n_copy], non_blocking=True)
+            h = self._decode_hidden(Bp)
+            flat = [i for i, r in enumerate(rows) if r]
+            self.stats["decode_steps"] += 1
+        else:
+            host = self._pack_prefill(batch, pad=True)
+            T, max_q = self.padded_tokens(batch.num_tokens), max(batch.num_query)
+            nd = B - len(batch.prefill_seqs) if self.split_mixed_attention else 0
+            buf = torch.from_numpy(host).to(self.device, non_blocking=False)
+            ids, meta, _ = self._prefill_meta(buf, T, B, max_q, len(batch.copies), nd, batch.num_tokens)
+            starts = np.concatenate([[0], np.cumsum(batch.num_query)])
+            flat_all = [int(starts[i]) + int(o) for i, r in enumerate(rows) for o in r]
+            meta.logits_indices = torch.tensor(flat_all, dtype=torch.int64, device=self.device)
+            prune = getattr(self.model, "prune_last_layer", None)
+            if prune is not None:   # Llama's last-layer row pruning assumes one sampled row per sequence
+                self.model.prune_last_layer = False
+            try:
+                h = self.model.forward(ids, meta, self.k_cache, self.v_cache)
+            finally:
+                if prune is not None:
+                    self.model.prune_last_layer = prune
+            flat = None
+            self.stats["prefill_steps"] += 1
+            self.stats["prefill_tokens"] += T
+        if flat is not None:
+            if not flat:
+                return torch.empty((0, self.cfg.vocab_size), dtype=torch.float32, device=self.device)
+            h = h.index_select(0, torch.tensor(flat, dtype=torch.int64, device=self.device))
+        elif h.shape[0] == 0:
+            return torch.empty((0, self.cfg.vocab_size), dtype=torch.float32, device=self.device)
+        return self.model.logits(h).float()
 
     # ------------------------------------------------------------------------------------------
     def _bcast_header(self, kind: int, a: int = 0, b: int = 0, c: int = 0, d: int = 0, e: int = 0,

@@ -270,6 +270,30 @@ class Scheduler:
                          partial=frozenset(partial))
         return Batch(decodes, [1] * len(decodes), is_decode=True)
 
+    def schedule_given(self, items: List[tuple]) -> Batch:
+        """A step whose composition the caller dictates (trace replay): items = [(sequence, n)] runs the
+        next n tokens of each sequence's `all_ids` from its `num_computed`.  Pages come from the block
+        manager as in `schedule` (all or nothing per row; NoFreeBlocks propagates), one-token rows of
+        sequences that already hold cache go first, as decode rows, and a step of only such rows is a
+        decode step.  The caller advances `num_computed` after the step and frees finished sequences
+        with `release`."""
+        dec, pre = [], []
+        for seq, n in items:
+            if n <= 0 or seq.num_computed + n > seq.total_len:
+                raise ValueError(f"seq {seq.seq_id}: {n} tokens from {seq.num_computed} of {seq.total_len}")
+            self.bm.ensure_capacity(seq.block_table, seq.num_computed + n)
+            seq.status = SeqStatus.RUNNING
+            (dec if n == 1 and seq.num_computed > 0 and seq.num_computed + 1 == seq.total_len else pre).append((seq, n))
+        if not pre:
+            return Batch([s for s, _ in dec], [1] * len(dec), is_decode=True)
+        return Batch([s for s, _ in dec + pre], [n for _, n in dec + pre], is_decode=False,
+                     prefill_seqs=[s for s, _ in pre])
+
+    def release(self, seq: Sequence) -> None:
+        """Give a sequence's pages back (a request that ends outside `on_step_done`)."""
+        self.bm.free_table(seq.block_table)
+        seq.status = SeqStatus.FINISHED
+
     def _preempt(self, seq: Sequence) -> None:
         """Recompute-style preemption: drop the KV, requeue; re-admission prefills all_ids."""
         self.running.remove(seq)

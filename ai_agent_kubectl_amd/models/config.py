@@ -7,7 +7,9 @@ same shape family used by CPU tests and GPU numerics tests.
 from __future__ import annotations
 
 import dataclasses
-from typing import Dict
+import json
+import os
+from typing import Dict, Optional, Tuple
 
 
 @dataclasses.dataclass(frozen=True)
@@ -65,6 +67,127 @@ class ModelConfig:
         return self.num_layers * 2 * self.kv_size * dtype_bytes
 
 
+@dataclasses.dataclass(frozen=True)
+class AttentionSpec:
+    """One attention mixer of a per-layer-configured model (the `mixer` entry of a Vivepel layer)."""
+    heads: int
+    kv_heads: int
+    dim: int                    # per-head query / key size
+    vdim: int                   # per-head value size (the values are the projected keys: vdim == dim)
+    chunk: int                  # chunked causal mask: position p sees floor(p / chunk) * chunk .. p
+    rot_dims: int               # rotary positions on the first rot_dims entries of each head
+    rot_base: float
+    scale: float
+    softcap: float
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "AttentionSpec":
+        spec = cls(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                   chunk=int(m["mask"]["size"]), rot_dims=int(m["rot"]["dims"]), rot_base=float(m["rot"]["base"]),
+                   scale=float(m["scale"]), softcap=float(m["softcap"]))
+        if spec.heads % spec.kv_heads:
+            raise ValueError(f"heads {spec.heads} must be a multiple of kv_heads {spec.kv_heads}")
+        if spec.vdim != spec.dim:
+            raise ValueError(f"vdim {spec.vdim} != dim {spec.dim}: the values are the projected keys")
+        if spec.rot_dims % 2 or spec.rot_dims > spec.dim or spec.chunk <= 0:
+            raise ValueError(f"bad rotary dims {spec.rot_dims} / chunk {spec.chunk} for head size {spec.dim}")
+        return spec
+
+
+@dataclasses.dataclass(frozen=True)
+class LayerSpec:
+    mixer: AttentionSpec
+    ff: int = 0                 # dense feed-forward width; 0: the layer has no feed-forward
+
+
+@dataclasses.dataclass(frozen=True)
+class VivepelConfig:
+    """Vivepel: a decoder whose layers are listed one by one in its config.json.  Every layer is
+    x += ls1 * gnorm(mixer(gnorm(x))), then (if it has one) x += ls2 * gnorm(ff(gnorm(x))), with RMS
+    norms in `norm_groups` groups; the mixer is chunk-masked attention (AttentionSpec), the
+    feed-forward is up -> PolyNorm -> down.  The residual stream is fp32."""
+    name: str
+    vocab_size: int
+    hidden: int
+    norm_eps: float
+    norm_groups: int
+    layers: Tuple[LayerSpec, ...]
+    max_position: int = 1 << 20
+    tokenizer: str = "llama3"
+    family: str = "vivepel"
+    tie_embeddings: bool = False
+    is_moe: bool = False
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_dict(cls, d: dict, name: str = "vivepel") -> "VivepelConfig":
+        layers = []
+        for i, L in enumerate(d["layers"]):
+            if L["type"] != "attention":
+                raise ValueError(f"layer {i}: unknown mixer type {L['type']!r}")
+            mlp = L.get("mlp")
+            if mlp is not None and mlp.get("kind") != "dense":
+                raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+            layers.append(LayerSpec(AttentionSpec.from_dict(L["mixer"]), int(mlp["ff"]) if mlp is not None else 0))
+        cfg = cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]), norm_eps=float(d["norm"]["eps"]),
+                  norm_groups=int(d["norm"]["groups"]), layers=tuple(layers))
+        if cfg.hidden % cfg.norm_groups:
+            raise ValueError(f"width {cfg.hidden} is not a multiple of norm groups {cfg.norm_groups}")
+        return cfg
+
+    def to_dict(self) -> dict:
+        """The config.json form (what `from_dict` reads)."""
+        return {"architecture": "Vivepel", "vocab": self.vocab_size, "width": self.hidden,
+                "norm": {"eps": self.norm_eps, "groups": self.norm_groups},
+                "layers": [{"type": "attention",
+                            "mixer": {"heads": L.mixer.heads, "kv_heads": L.mixer.kv_heads, "dim": L.mixer.dim,
+                                      "vdim": L.mixer.vdim, "mask": {"size": L.mixer.chunk},
+                                      "rot": {"base": L.mixer.rot_base, "dims": L.mixer.rot_dims},
+                                      "scale": L.mixer.scale, "softcap": L.mixer.softcap},
+                            "mlp": {"kind": "dense", "ff": L.ff} if L.ff else None} for L in self.layers]}
+
+    def num_params(self) -> int:
+        h = self.hidden
+        n = 2 * self.vocab_size * h + h
+        for L in self.layers:
+            m = L.mixer
+            n += (m.heads + m.kv_heads) * m.dim * (h + 1) + m.heads * m.vdim * h + m.heads * m.heads + 2 * m.dim + 3 * h
+            if L.ff:
+                n += 2 * h * L.ff + 4 + 3 * h
+        return n
+
+    def default_step_tokens(self) -> int:
+        return 4096
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        return sum(2 * L.mixer.kv_heads * L.mixer.dim * dtype_bytes for L in self.layers)
+
+
+def vivepel_uniform(name: str, layers: int, hidden: int, heads: int, kv_heads: int, dim: int, ff: int, vocab: int,
+                    chunk: int = 1024, rot_dims: Optional[int] = None, groups: int = 4) -> VivepelConfig:
+    """A Vivepel configuration whose layers are all alike (benchmarks, tests)."""
+    spec = AttentionSpec(heads, kv_heads, dim, dim, chunk, rot_dims if rot_dims is not None else dim // 2, 10000.0,
+                         dim ** -0.5, 30.0)
+    return VivepelConfig(name, vocab, hidden, 1e-6, groups, tuple(LayerSpec(spec, ff) for _ in range(layers)))
+
+
+# config.json "architecture" -> parser of the file's dict
+ARCHITECTURES = {"Vivepel": VivepelConfig.from_dict}
+
+
+def load_config_dir(path: str):
+    """The configuration of a checkpoint folder (config.json + model.safetensors), by its architecture."""
+    with open(os.path.join(path, "config.json")) as f:
+        d = json.load(f)
+    arch = d.get("architecture")
+    if arch not in ARCHITECTURES:
+        raise ValueError(f"{path}/config.json: unknown architecture {arch!r}; known: {sorted(ARCHITECTURES)}")
+    return ARCHITECTURES[arch](d, name=os.path.basename(os.path.normpath(path)) or arch.lower())
+
+
 PRESETS: Dict[str, ModelConfig] = {
     "llama3-8b": ModelConfig("llama3-8b", "llama", 32, 4096, 32, 8, 128, 14336, 128256, 500000.0),
     "llama3-70b": ModelConfig("llama3-70b", "llama", 80, 8192, 64, 8, 128, 28672, 128256, 500000.0),
@@ -86,11 +209,17 @@ PRESETS: Dict[str, ModelConfig] = {
     "llama3-70b-tiny": ModelConfig("llama3-70b-tiny", "llama", 2, 2048, 64, 8, 32, 1024, 128256, 500000.0),
     "mixtral-2l": ModelConfig("mixtral-2l", "mixtral", 2, 4096, 32, 8, 128, 14336, 32000, 1e6, max_position=32768,
                               num_experts=8, top_k=2, tokenizer="llama2"),
+    # Vivepel at small sizes (CPU tests) and at the layer sizes of Llama-3-8B (bench.py --arch-compare)
+    "tiny-vivepel": vivepel_uniform("tiny-vivepel", 2, 128, 4, 2, 32, 192, 384, chunk=16, rot_dims=12, groups=2),
+    "vivepel-8b-2l": vivepel_uniform("vivepel-8b-2l", 2, 4096, 32, 8, 128, 14336, 128256),
+    "vivepel-8b": vivepel_uniform("vivepel-8b", 32, 4096, 32, 8, 128, 14336, 128256),
 }
 
 
-def get_config(name: str) -> ModelConfig:
-    try:
+def get_config(name: str):
+    """A preset by name, or a checkpoint folder (its config.json names the architecture)."""
+    if name in PRESETS:
         return PRESETS[name]
-    except KeyError:
-        raise ValueError(f"unknown MODEL {name!r}; choose from {sorted(PRESETS)}") from None
+    if os.path.isdir(name) and os.path.exists(os.path.join(name, "config.json")):
+        return load_config_dir(name)
+    raise ValueError(f"unknown MODEL {name!r}; choose from {sorted(PRESETS)} or give a checkpoint folder")

@@ -111,6 +111,16 @@ class LlamaModel:
         self._pd_max_b = None
         self.persistent_stamps = None   # diagnostics: int64 [CUs, L, 16] phase timestamps (scripts/)
 
+    supports_block_copy = True   # ops.kv_block_copy knows this cache layout (sub-block prefix reuse)
+
+    def alloc_cache(self, num_blocks: int, block_size: int):
+        """(k_cache [L, NB, Hkv, BS, D], v_cache [L, NB, Hkv, D, BS]) for this rank's KV heads, zero-filled:
+        stale slots read by masked lanes must be finite (attention.hip contract)."""
+        L, dt = self.cfg.num_layers, self.W["embed"].dtype
+        k = torch.zeros((L, num_blocks, self.hkv, block_size, self.D), dtype=dt, device=self.device)
+        v = torch.zeros((L, num_blocks, self.hkv, self.D, block_size), dtype=dt, device=self.device)
+        return k, v
+
     def _layer(self, i):
         p = f"layers.{i}."
         return {k: self.W[p + k] for k in ("wqkv", "wo", "ln1", "ln2", "w13", "w2", "router") if p + k in self.W}

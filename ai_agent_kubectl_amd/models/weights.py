@@ -193,7 +193,129 @@ def load_safetensors(path: str, cfg: ModelConfig, par: ParallelInfo, device="cpu
     return {k: v.to(device=device, dtype=dtype).contiguous() for k, v in W.items()}
 
 
+# ------------------------------------------------------------------------------------------------
+# Vivepel.  Engine layout per layer `layers.<i>.`: wqk [(H + G) * D, W] with bias bqk (the q rows, then
+# the k rows: one GEMM), wo [W, H * Dv], w_up [ff, W], w_down [W, ff] in the activation dtype; the
+# norm weights (norm1, norm1b, norm2, norm2b, q_norm, k_norm), the layer scales (ls1, ls2), the head
+# mixing matrix (talk), the PolyNorm coefficients (act) and the rotary frequencies (inv_freq) in fp32,
+# because the ops that read them compute in fp32.
+_VIVEPEL_F32 = ("norm1", "norm1b", "norm2", "norm2b", "ls1", "ls2", "q_norm", "k_norm", "talk", "act", "inv_freq")
+
+
+def _vivepel_pack(cfg, get, device, dtype) -> Dict[str, torch.Tensor]:
+    """get(checkpoint name) -> tensor; returns the engine layout on `device`."""
+    W: Dict[str, torch.Tensor] = {"embed": get("embed"), "lm_head": get("head"), "norm": get("final.norm").float()}
+    for i, L in enumerate(cfg.layers):
+        p, c, m = f"layers.{i}.", f"l{i}.", L.mixer
+        W[p + "wqk"] = torch.cat([get(c + "mix.q"), get(c + "mix.k")])
+        W[p + "bqk"] = torch.cat([get(c + "mix.q.b"), get(c + "mix.k.b")])
+        W[p + "wo"] = get(c + "mix.o")
+        W[p + "q_norm"], W[p + "k_norm"] = get(c + "mix.q.norm"), get(c + "mix.k.norm")
+        W[p + "talk"] = get(c + "mix.talk")
+        for k in ("norm1", "norm1b", "ls1"):
+            W[p + k] = get(c + k)
+        half = m.rot_dims // 2
+        # base^(-2i / dims) in float64, rounded once to fp32; the angle is position * inv_freq in fp32
+        W[p + "inv_freq"] = (float(m.rot_base) ** (-2.0 * torch.arange(half, dtype=torch.float64) / max(m.rot_dims, 1)))
+        if L.ff:
+            W[p + "w_up"], W[p + "w_down"], W[p + "act"] = get(c + "mlp.up"), get(c + "mlp.down"), get(c + "mlp.act")
+            for k in ("norm2", "norm2b", "ls2"):
+                W[p + k] = get(c + k)
+    out = {}
+    for k, v in W.items():
+        f32 = k == "norm" or k.rsplit(".", 1)[-1] in _VIVEPEL_F32
+        out[k] = v.to(device=device, dtype=torch.float32 if f32 else dtype).contiguous()
+    return out
+
+
+def vivepel_check_shapes(cfg, W: Dict[str, torch.Tensor]) -> None:
+    """Every tensor of the engine layout has the shape the configuration implies."""
+    h, V = cfg.hidden, cfg.vocab_size
+    want = {"embed": (V, h), "lm_head": (V, h), "norm": (h,)}
+    for i, L in enumerate(cfg.layers):
+        p, m = f"layers.{i}.", L.mixer
+        n = (m.heads + m.kv_heads) * m.dim
+        want.update({p + "wqk": (n, h), p + "bqk": (n,), p + "wo": (h, m.heads * m.vdim), p + "q_norm": (m.dim,),
+                     p + "k_norm": (m.dim,), p + "talk": (m.heads, m.heads), p + "norm1": (h,), p + "norm1b": (h,),
+                     p + "ls1": (h,), p + "inv_freq": (m.rot_dims // 2,)})
+        if L.ff:
+            want.update({p + "w_up": (L.ff, h), p + "w_down": (h, L.ff), p + "act": (4,), p + "norm2": (h,),
+                         p + "norm2b": (h,), p + "ls2": (h,)})
+    for k, shp in want.items():
+        if k not in W or tuple(W[k].shape) != shp:
+            raise ValueError(f"tensor {k}: expected shape {shp}, found {tuple(W[k].shape) if k in W else None}")
+
+
+def vivepel_checkpoint_tensors(cfg, seed: int = 0, dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Random tensors under the checkpoint's own names (what a Vivepel model.safetensors holds)."""
+    g = torch.Generator().manual_seed(_seed(seed, "vivepel") & 0x7FFFFFFF)
+    h, V = cfg.hidden, cfg.vocab_size
+
+    def mat(o, i, std=None):
+        return (torch.randn(o, i, generator=g) * (std if std is not None else i ** -0.5)).to(dtype)
+
+    def vec(n, lo=0.75, hi=1.25):
+        return (lo + (hi - lo) * torch.rand(n, generator=g)).to(dtype)
+
+    T = {"embed": mat(V, h, 1.0), "head": mat(V, h), "final.norm": vec(h)}
+    for i, L in enumerate(cfg.layers):
+        c, m = f"l{i}.", L.mixer
+        T[c + "mix.q"], T[c + "mix.q.b"] = mat(m.heads * m.dim, h), (torch.randn(m.heads * m.dim, generator=g) * 0.1).to(dtype)
+        T[c + "mix.k"], T[c + "mix.k.b"] = mat(m.kv_heads * m.dim, h), (torch.randn(m.kv_heads * m.dim, generator=g) * 0.1).to(dtype)
+        T[c + "mix.q.norm"], T[c + "mix.k.norm"] = vec(m.dim), vec(m.dim)
+        T[c + "mix.talk"] = (torch.eye(m.heads) * 0.8 + torch.randn(m.heads, m.heads, generator=g) * (0.2 / m.heads ** 0.5)).to(dtype)
+        T[c + "mix.o"] = mat(h, m.heads * m.vdim)
+        for k in ("norm1", "norm1b"):
+            T[c + k] = vec(h)
+        T[c + "ls1"] = vec(h, 0.2, 0.6)
+        if L.ff:
+            T[c + "mlp.up"], T[c + "mlp.down"] = mat(L.ff, h), mat(h, L.ff)
+            T[c + "mlp.act"] = torch.tensor([0.6, 0.3, 0.15, 0.02]).to(dtype)
+            for k in ("norm2", "norm2b"):
+                T[c + k] = vec(h)
+            T[c + "ls2"] = vec(h, 0.2, 0.6)
+    return T
+
+
+def vivepel_random_weights(cfg, seed: int = 0, device="cpu", dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Random-init Vivepel weights: drawn in bf16 (as a checkpoint stores them), packed for `dtype`."""
+    T = vivepel_checkpoint_tensors(cfg, seed)
+    W = _vivepel_pack(cfg, T.__getitem__, device, dtype)
+    vivepel_check_shapes(cfg, W)
+    return W
+
+
+def load_vivepel_safetensors(path: str, cfg, device="cpu", dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """A Vivepel checkpoint (a file, or a folder holding model.safetensors / *.safetensors)."""
+    from safetensors import safe_open
+
+    files = [path] if os.path.isfile(path) else sorted(glob.glob(os.path.join(path, "*.safetensors")))
+    if not files:
+        raise FileNotFoundError(f"no .safetensors under {path}")
+    index = {}
+    for f in files:
+        hnd = safe_open(f, framework="pt", device="cpu")
+        for k in hnd.keys():
+            index[k] = hnd
+
+    def get(name):
+        if name not in index:
+            raise KeyError(f"{path}: tensor {name!r} is missing")
+        return index[name].get_tensor(name)
+
+    W = _vivepel_pack(cfg, get, device, dtype)
+    vivepel_check_shapes(cfg, W)
+    return W
+
+
 def build_weights(spec: str, cfg: ModelConfig, par: ParallelInfo, device="cpu", dtype=torch.bfloat16):
+    if getattr(cfg, "family", "") == "vivepel":
+        if par.tp_size != 1 or par.ep_size != 1:
+            raise ValueError("Vivepel runs at TP = 1 (data parallel replicas scale it out)")
+        if spec.startswith("random"):
+            seed = int(spec.split(":", 1)[1]) if ":" in spec else 0
+            return vivepel_random_weights(cfg, seed=seed, device=device, dtype=dtype)
+        return load_vivepel_safetensors(spec, cfg, device=device, dtype=dtype)
     if spec.startswith("random"):
         seed = int(spec.split(":", 1)[1]) if ":" in spec else 0
         return random_weights(cfg, par, seed=seed, device=device, dtype=dtype)

@@ -106,6 +106,35 @@ _SIGS = {
 }
 
 
+_MIX_SIGS = {
+    "ka_embed_f32": [P, P, P, I, I, I, I, P],
+    "ka_group_rmsnorm": [P, P, P, I, I, I, F, I, I, P],
+    "ka_post_norm_residual": [P, P, P, P, P, P, I, I, I, F, I, P],
+    "ka_polynorm": [P, P, P, I, I, F, I, P],
+    "ka_headnorm_rope_append": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, P],
+    "ka_chunk_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, F, I, P],
+}
+MIXERS_LIB = os.path.join(LIB_DIR, "libkagent_mixers.so")
+_mix: Optional[ctypes.CDLL] = None
+
+
+def require_mixers() -> ctypes.CDLL:
+    """The small library of the fp32-residual models' kernels (build.build_mixers); raises if it is not built."""
+    global _mix
+    with _lock:
+        if _mix is None:
+            if not os.path.exists(MIXERS_LIB):
+                raise RuntimeError(f"HIP kernel library not built: {MIXERS_LIB} "
+                                   "(run python -c 'import __graft_entry__ as g; g.build()')")
+            lib = ctypes.CDLL(MIXERS_LIB, mode=ctypes.RTLD_GLOBAL)
+            for name, argtypes in _MIX_SIGS.items():
+                fn = getattr(lib, name)
+                fn.argtypes = argtypes
+                fn.restype = ctypes.c_int
+            _mix = lib
+        return _mix
+
+
 def load(path: str = LIB_PATH) -> Optional[ctypes.CDLL]:
     """Load the library once; returns None (and remembers why) if it is missing."""
     global _lib, _err

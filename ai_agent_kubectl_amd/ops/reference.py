@@ -144,3 +144,95 @@ def argmax_combine(vals: torch.Tensor, idxs: torch.Tensor) -> torch.Tensor:
     big = torch.iinfo(torch.int32).max
     cand = torch.where(v == best, idxs.to(torch.int64), torch.full_like(idxs, big, dtype=torch.int64))
     return cand.min(dim=0).values.to(torch.int32)
+
+
+# ------------------------------------------------------------------------------------------------
+# fp32-residual models (models/vivepel.py): the ops of ops/mixers.py on CPU tensors.  Statistics,
+# scores and weights in fp32; outputs in the activation dtype.
+def group_rmsnorm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float, out_dtype=None) -> torch.Tensor:
+    """Row cut into `groups` equal parts, each divided by sqrt(mean(part^2) + eps); times w."""
+    xf = x.float()
+    parts = xf.view(xf.shape[0], groups, -1)
+    y = (parts / torch.sqrt(parts.pow(2).mean(-1, keepdim=True) + eps)).view_as(xf) * w.float()
+    return y.to(out_dtype or x.dtype)
+
+
+def post_norm_residual(resid, y, w_post, ls, w_next, groups: int, eps: float):
+    """resid += ls * gnorm(y; w_post) (in place, fp32); returns gnorm(resid; w_next) in y's dtype, or None."""
+    resid.add_(ls.float() * group_rmsnorm(y, w_post, groups, eps, torch.float32))
+    return group_rmsnorm(resid, w_next, groups, eps, y.dtype) if w_next is not None else None
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    zf = z.float()
+    z2 = zf * zf
+
+    def n(u):
+        return u / torch.sqrt(u.pow(2).mean(-1, keepdim=True) + eps)
+
+    c = coef.float()
+    return (c[0] * n(zf) + c[1] * n(z2) + c[2] * n(z2 * zf) + c[3]).to(z.dtype)
+
+
+def headnorm_rope_append(qk, q_w, k_w, inv_freq, positions, slots, k_cache, v_cache, H: int, G: int, D: int,
+                         rot: int, eps: float):
+    """qk [T, (H + G) * D] -> q [T, H, D] normed + rotated; the normed + rotated keys and the raw keys
+    (the values) go to k_cache / v_cache [NB, G, BS, D] at `slots`."""
+    T = qk.shape[0]
+    x = qk.view(T, H + G, D)
+    xf = x.float()
+    w = torch.cat([q_w.float().expand(H, D), k_w.float().expand(G, D)])
+    y = xf / torch.sqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w
+    half = rot // 2
+    if half:
+        ang = positions.float()[:, None] * inv_freq.float()[None, :]
+        cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        a, b = y[..., :half], y[..., half:rot]
+        y = torch.cat([a * cos - b * sin, b * cos + a * sin, y[..., rot:]], dim=-1)
+    y = y.to(qk.dtype)
+    bs = k_cache.shape[2]
+    s = slots.long()
+    ok = s >= 0
+    if ok.any():
+        k_cache[s[ok] // bs, :, s[ok] % bs, :] = y[ok][:, H:]
+        v_cache[s[ok] // bs, :, s[ok] % bs, :] = x[ok][:, H:]
+    return y[:, :H].contiguous()
+
+
+def chunk_attention(q, k_cache, v_cache, block_tables, q_starts, positions, slots, mix, chunk: int, scale: float,
+                    cap: float, sink: bool):
+    """q [T, H, D] -> [T, H * Dv]; see csrc/attention_chunk.hip for the options."""
+    T, H, D = q.shape
+    G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    rep = H // G
+    out = torch.zeros(T, H * Dv, dtype=q.dtype, device=q.device)
+    pos_l, slot_l = positions.tolist(), slots.tolist()
+    seq_l = list(range(T))
+    if q_starts is not None:
+        qs = q_starts.tolist()
+        seq_l = [0] * T
+        for i in range(len(qs) - 1):
+            seq_l[qs[i]:qs[i + 1]] = [i] * (qs[i + 1] - qs[i])
+    for t in range(T):
+        if slot_l[t] < 0:
+            continue
+        p = pos_l[t]
+        start = (p // chunk) * chunk if chunk > 0 else 0
+        js = torch.arange(start, p + 1, device=q.device)
+        pages = block_tables[seq_l[t]].long()[js // bs]
+        k = k_cache[pages, :, js % bs, :].float()             # [n, G, D]
+        v = v_cache[pages, :, js % bs, :].float()             # [n, G, Dv]
+        k = k.repeat_interleave(rep, dim=1)                   # [n, H, D]
+        s = torch.einsum("hd,nhd->hn", q[t].float(), k) * scale
+        if cap > 0:
+            s = cap * torch.tanh(s / cap)
+        m = s.max(dim=1, keepdim=True).values
+        if sink:
+            m = m.clamp(min=0.0)
+        e = torch.exp(s - m)
+        w = e / (e.sum(dim=1, keepdim=True) + (torch.exp(-m) if sink else 0.0))
+        if mix is not None:
+            w = mix.float() @ w
+        o = torch.einsum("hn,nhd->hd", w, v.repeat_interleave(rep, dim=1))
+        out[t] = o.reshape(-1).to(q.dtype)
+    return out
