@@ -152,7 +152,7 @@ def argmax_combine(vals: torch.Tensor, idxs: torch.Tensor) -> torch.Tensor:
 def group_rmsnorm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float, out_dtype=None) -> torch.Tensor:
     """Row cut into `groups` equal parts, each divided by sqrt(mean(part^2) + eps); times w."""
     xf = x.float()
-    parts = xf.view(xf.shape[0], groups, -1)
+    parts = xf.view(xf.shape[0], groups, xf.shape[1] // groups)
     y = (parts / torch.sqrt(parts.pow(2).mean(-1, keepdim=True) + eps)).view_as(xf) * w.float()
     return y.to(out_dtype or x.dtype)
 

@@ -132,6 +132,14 @@ def parse_args(argv=None):
                     help="tensor-parallel degree of each engine replica (BASELINE configs #3 / #4: "
                          "--model llama3-70b --tp 8, --model mixtral-8x7b --tp 8 = EP 8); the server runs "
                          "DP = gpus / tp replicas, each a TP group of consecutive GPUs (tcp transport)")
+    ap.add_argument("--arch-compare", action="store_true",
+                    help="instead of the headline workload: engine prefill / decode tokens/s of Vivepel beside "
+                         "Llama at equal layer sizes (ai_agent_kubectl_amd/bench_arch.py); one JSON line")
+    ap.add_argument("--arch-sizes", default="2k,8b", help="--arch-compare: sizes of bench_arch.SIZES, comma-separated")
+    ap.add_argument("--arch-batch", type=int, default=32)
+    ap.add_argument("--arch-prompt", type=int, default=1024)
+    ap.add_argument("--arch-chunk", type=int, default=1024, help="--arch-compare: Vivepel's attention chunk")
+    ap.add_argument("--arch-models", default="llama,vivepel")
     args = ap.parse_args(argv)
     if args.tp < 1 or args.gpus % args.tp:
         ap.error(f"--tp {args.tp} must divide --gpus {args.gpus}")
@@ -714,6 +722,11 @@ def run_asgi(args, rank, local, world, C, buckets, dist, prefix_caching=True):
 
 def main():
     args = parse_args()
+    if args.arch_compare:
+        from ai_agent_kubectl_amd import bench_arch
+        print(json.dumps(bench_arch.main(tuple(args.arch_sizes.split(",")), args.arch_batch, args.arch_prompt,
+                                         args.max_new_tokens * 2, args.arch_chunk, tuple(args.arch_models.split(",")))))
+        return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         # `python bench.py --gpus N`: spawn the N ranks ourselves, before anything touches a GPU,
         # as a child torch.distributed.run job (one process per GPU), and exit with its status
