@@ -21,7 +21,7 @@
 // head's weight for a key in one place).  Pass 1 finds each head's maximum and denominator over the
 // visible keys, pass 2 recomputes the scores tile by tile, normalises, mixes the heads and
 // accumulates weights x values.  A decode step is the same launch with one token per sequence.
-#include "common.h"
+#include "attention_chunk.h"
 
 namespace {
 
@@ -102,16 +102,6 @@ __global__ __launch_bounds__(NT) void headnorm_rope_append_kernel(
   }
 }
 
-struct AttnArgs {
-  const int* block_tables;   // [S, max_blocks]
-  const int* q_starts;       // [S + 1] first token of each sequence's rows (varlen step); null: token t is row t
-  int num_seqs;
-  const int* positions;      // [T]
-  const int* slots;          // [T]  < 0: padding row
-  const float* mix;          // [H, H] or null
-  int H, G, D, Dv, chunk, BS, max_blocks, sink;
-  float scale, cap;
-};
 
 template <typename AT>
 __global__ __launch_bounds__(NT) void chunk_attention_kernel(AT* __restrict__ out, const AT* __restrict__ q,
@@ -161,7 +151,28 @@ __global__ __launch_bounds__(NT) void chunk_attention_kernel(AT* __restrict__ ou
     const AT* kr = k_cache + (((size_t)page[j - (j / KT) * KT] * G + g / rep) * BS + pos % BS) * D;
     const float* qg = qs + g * D;
     float s = 0.f;
-    for (int i = 0; i < D; ++i) s += qg[i] * ldf(kr + i);
+    if constexpr (sizeof(AT) == 2) {
+      if ((D & 7) == 0) {   // 16-byte loads: 8 bf16 keys entries against 8 fp32 query entries from LDS
+        for (int i = 0; i < D; i += 8) {
+          const uint4 kv = *reinterpret_cast<const uint4*>(kr + i);
+          const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + i), qb = *reinterpret_cast<const f32x4*>(qg + i + 4);
+          s += qa[0] * lo_f(kv.x) + qa[1] * hi_f(kv.x) + qa[2] * lo_f(kv.y) + qa[3] * hi_f(kv.y) +
+               qb[0] * lo_f(kv.z) + qb[1] * hi_f(kv.z) + qb[2] * lo_f(kv.w) + qb[3] * hi_f(kv.w);
+        }
+      } else {
+        for (int i = 0; i < D; ++i) s += qg[i] * ldf(kr + i);
+      }
+    } else {
+      if ((D & 3) == 0) {
+        for (int i = 0; i < D; i += 4) {
+          const f32x4 kv = *reinterpret_cast<const f32x4*>(kr + i);
+          const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + i);
+          s += qa[0] * kv[0] + qa[1] * kv[1] + qa[2] * kv[2] + qa[3] * kv[3];
+        }
+      } else {
+        for (int i = 0; i < D; ++i) s += qg[i] * ldf(kr + i);
+      }
+    }
     s *= a.scale;
     return a.cap > 0.f ? a.cap * tanhf(s / a.cap) : s;
   };

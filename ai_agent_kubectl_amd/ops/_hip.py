@@ -113,6 +113,8 @@ _MIX_SIGS = {
     "ka_polynorm": [P, P, P, I, I, F, I, P],
     "ka_headnorm_rope_append": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, P],
     "ka_chunk_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, F, I, P],
+    "ka_chunk_attention_tile_ok": [I, I, I, I, I],
+    "ka_chunk_attention_tile": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, F, P],
 }
 MIXERS_LIB = os.path.join(LIB_DIR, "libkagent_mixers.so")
 _mix: Optional[ctypes.CDLL] = None

@@ -17,6 +17,9 @@ from . import reference as ref
 from ._hip import check, require_mixers
 
 
+TILE_MIN_Q = 8   # varlen steps whose longest row run is shorter stay on the per-token attention kernel
+
+
 def _ref(t: torch.Tensor) -> bool:
     from . import _FORCE_REF
     return _FORCE_REF or not t.is_cuda
@@ -114,7 +117,8 @@ def headnorm_rope_append(qk: torch.Tensor, q_w: torch.Tensor, k_w: torch.Tensor,
 
 def chunk_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     q_starts: Optional[torch.Tensor], positions: torch.Tensor, slots: torch.Tensor,
-                    mix: Optional[torch.Tensor], chunk: int, scale: float, cap: float, sink: bool) -> torch.Tensor:
+                    mix: Optional[torch.Tensor], chunk: int, scale: float, cap: float, sink: bool,
+                    max_q: int = 0) -> torch.Tensor:
     """q [T, H, D] -> [T, H * Dv].  q_starts [S + 1]: first row of each sequence in a varlen step (rows
     past q_starts[S] must be padding, slot < 0); None: token t is block-table row t (a decode step).  chunk 0: plain causal; cap 0: no soft cap; mix None: no head mixing."""
     if _ref(q):
@@ -129,6 +133,15 @@ def chunk_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     assert q_starts is None or (q_starts.dtype == torch.int32 and q_starts.shape[0] == block_tables.shape[0] + 1)
     assert q_starts is not None or block_tables.shape[0] >= T
     assert mix is None or (mix.dtype == torch.float32 and mix.shape == (H, H) and mix.is_contiguous())
+    if (q_starts is not None and max_q >= TILE_MIN_Q and q.dtype == torch.bfloat16
+            and lib.ka_chunk_attention_tile_ok(H, G, D, Dv, BS)):
+        # rows past the last sequence (a padded step) belong to no tile: they stay zero
+        out = torch.zeros((T, H * Dv), dtype=q.dtype, device=q.device)
+        check(lib.ka_chunk_attention_tile(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(q_starts),
+                                          block_tables.shape[0], _p(positions), _p(slots), _p(mix), int(max_q), H, G, D,
+                                          Dv, int(chunk), BS, block_tables.shape[1], int(bool(sink)), float(scale),
+                                          float(cap), _stream()), "chunk_attention_tile")
+        return out
     out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
     check(lib.ka_chunk_attention(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(q_starts),
                                  block_tables.shape[0], _p(positions), _p(slots), _p(mix), T, H, G, D, Dv, int(chunk), BS,

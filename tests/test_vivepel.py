@@ -183,7 +183,8 @@ def test_headnorm_rope_append(device, H, G, D, rot):
         assert torch.equal(vc[page, :, off].cpu(), x[t, H:])      # the value is the key as projected
 
 
-def _attention_case(device, H, G, D, chunk, cap, sink, mix, positions_q, n_ctx, bs=4, seed=0, q=None, k=None, v=None):
+def _attention_case(device, H, G, D, chunk, cap, sink, mix, positions_q, n_ctx, bs=4, seed=0, q=None, k=None, v=None,
+                    dtype=torch.float32, max_q=0):
     """chunk_attention for queries at `positions_q` of one sequence holding n_ctx cached tokens, against
     a direct evaluation; returns (got, want)."""
     from ai_agent_kubectl_amd.ops import mixers
@@ -193,6 +194,7 @@ def _attention_case(device, H, G, D, chunk, cap, sink, mix, positions_q, n_ctx, 
     k = torch.randn(n_ctx, G, D, generator=g) if k is None else k
     v = torch.randn(n_ctx, G, D, generator=g) if v is None else v
     q = torch.randn(len(positions_q), H, D, generator=g) if q is None else q
+    q, k, v = (t.to(dtype).float() for t in (q, k, v))                            # what the kernel's dtype can hold
     kc, vc = torch.full((nb, G, bs, D), 1e3), torch.full((nb, G, bs, D), 1e3)    # unused slots: loud if read
     for j in range(n_ctx):
         kc[table[j // bs], :, j % bs] = k[j]
@@ -206,9 +208,10 @@ def _attention_case(device, H, G, D, chunk, cap, sink, mix, positions_q, n_ctx, 
         q_starts = None
     else:
         q_starts = torch.tensor([0, T], dtype=torch.int32)
-    got = mixers.chunk_attention(q.to(device), kc.to(device), vc.to(device), bt.to(device),
+    got = mixers.chunk_attention(q.to(device, dtype), kc.to(device, dtype), vc.to(device, dtype), bt.to(device),
                                  None if q_starts is None else q_starts.to(device), pos.to(device), slots.to(device),
-                                 None if mix is None else mix.to(device), chunk, scale, cap, sink).cpu()
+                                 None if mix is None else mix.to(device), chunk, scale, cap, sink,
+                                 max_q=max_q).float().cpu()
     rep = H // G
     want = torch.zeros(T, H, D)
     for t, p in enumerate(positions_q):
@@ -240,6 +243,26 @@ def test_chunk_attention_options(device, H, G, D, chunk, cap, sink, mixed):
             continue
         got, want = _attention_case(device, H, G, D, chunk, cap, sink, mix, [p], n)
         assert torch.allclose(got, want, rtol=1e-4, atol=1e-4), p
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,chunk,cap,sink,mixed", [(6, 2, 96, 48, 50.0, True, True), (20, 4, 32, 24, 0.0, True, True),
+                                                        (32, 8, 128, 40, 30.0, True, True), (3, 1, 64, 0, 5.0, False, False),
+                                                        (5, 5, 32, 7, 9.0, True, True), (17, 17, 64, 1000, 20.0, True, True)])
+def test_chunk_attention_tile_kernel(H, G, D, chunk, cap, sink, mixed):
+    """bf16 prompt portions on the 16-row tile kernel (MFMA scores): portions that start and end inside
+    chunks, pages and 16-row tiles, against the direct fp32 evaluation of the same bf16 inputs."""
+    from ai_agent_kubectl_amd.ops import _hip
+
+    assert _hip.require_mixers().ka_chunk_attention_tile_ok(H, G, D, D, 4) == 1
+    mix = (torch.eye(H) * 0.6 + torch.randn(H, H, generator=torch.Generator().manual_seed(9)) * (0.4 / H ** 0.5)) if mixed else None
+    for lo, n in ((0, 70), (37, 90), (63, 81), (5, 14)):
+        got, want = _attention_case("cuda", H, G, D, chunk, cap, sink, mix, list(range(lo, n)), n, dtype=torch.bfloat16,
+                                    max_q=n - lo, seed=lo)
+        assert torch.allclose(got, want, rtol=2e-2, atol=2e-2), (lo, n, float((got - want).abs().max()))
+        # the per-token kernel on the same inputs agrees too (max_q 0 keeps it off the tile kernel)
+        got1, _ = _attention_case("cuda", H, G, D, chunk, cap, sink, mix, list(range(lo, n)), n, dtype=torch.bfloat16, seed=lo)
+        assert torch.allclose(got, got1, rtol=2e-2, atol=2e-2)
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -435,6 +458,20 @@ def test_bf16_engine(tmp_path, name):
     want = want_logits(config, W, toks)
     assert rel_err(replay(sess, toks, [len(toks)]), want) < tol("bfloat16")
     assert rel_err(replay(sess, toks, [3, 2, 20] + [1] * 25), want) < tol("bfloat16")
+
+
+@pytest.mark.gpu
+def test_bf16_engine_tile_kernel_shapes(tmp_path):
+    """Head size 32 and portions of 8 rows and more: the engine's bf16 prompt steps run the tile kernel."""
+    g = torch.Generator().manual_seed(2)
+    config = oracle.random_config(g, layers=2, width=64, vocab=272, groups=2, heads=6, kv_heads=2, dim=32, vdim=32,
+                                  rot={"base": 1000.0, "dims": 20}, mask={"size": 24}, scale=0.2, softcap=15.0)
+    W = oracle.random_weights(config, seed=21)
+    sess = session(write_checkpoint(tmp_path / "m", config, W), "cuda", dtype="bfloat16")
+    toks = tokens_for(config, 75, seed=9)
+    want = want_logits(config, W, toks)
+    assert rel_err(replay(sess, toks, [len(toks)]), want) < tol("bfloat16")
+    assert rel_err(replay(sess, toks, [9, 17, 30, 2, 16, 1]), want) < tol("bfloat16")
 
 
 @pytest.mark.gpu
