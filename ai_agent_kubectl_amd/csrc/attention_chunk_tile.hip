@@ -1,32 +1,34 @@
 // KA_HIP_LIB: mixers
 // KA_HIPCC_FLAGS: -Xclang -target-feature -Xclang -packed-fp32-ops
-// Chunk-masked attention for prompt portions (bf16 activations and cache): one workgroup of 16 waves
+// Chunk-masked attention for prompt portions (bf16 activations and cache): one workgroup of 8 waves
 // per (sequence, 16 consecutive query rows) with ALL heads, because the head mixing needs every
 // head's weight of a (row, key) pair in one place before any value is touched.
 //
-//   scores     S_g = Q_g K_c(g)^T on MFMA 16x16x32 (bf16 in, fp32 out): wave w owns the heads w, w + 16, ...;
+//   scores     S_g = Q_g K_c(g)^T on MFMA 16x16x32 (bf16 in, fp32 out): wave w owns the heads w, w + 8, ...;
 //              its Q fragments stay in registers, the K fragments are 16-byte loads straight from the
 //              token-major pages (lane = key, 8 consecutive head entries), no LDS staging;
 //   pass 1     per head and row, the running maximum and denominator over the row's visible keys
 //              (soft cap, chunk mask, sink), kept in LDS as (maximum, 1 / denominator);
 //   pass 2     per tile of 16 keys: the normalised fp32 weights of all heads go to LDS, are mixed over
-//              the heads (mix[h, g] read as wave-uniform scalars), and each thread adds weight x value
-//              for 16 rows x 4 consecutive value entries of one head in fp32 registers.
-// Weights, mixing and the weights x values sums are fp32 on the vector ALUs (the weights are never
-// rounded to bf16); only Q K^T runs on the matrix cores, where bf16 inputs lose nothing.
+//              the heads, and multiplied with the values, both on the fp32 matrix instruction
+//              (mfma 16x16x4 f32): the weights are never rounded to bf16, the bf16 values are widened.
+// Only Q K^T runs at the bf16 MFMA rate, where bf16 inputs lose nothing; everything that the design
+// wants in 32 bits runs at the fp32 matrix rate (1/16 of the bf16 rate), which is this kernel's roofline.
+// A decode step (q_starts null) runs the same kernel with one row per workgroup: scores on MFMA with
+// one useful row, mixing and weights x values for that row on the vector ALUs.
 //
 // Shapes it takes (the launcher returns hipErrorInvalidValue otherwise and the caller uses the
-// per-token kernel): D a multiple of 32 up to 256, H <= 64, H * Dv <= 4096, Dv a multiple of 4.
+// per-token kernel): D a multiple of 32 up to 256, Dv == D, H <= 64, heads per wave x D <= 512.
 #include "attention_chunk.h"
 
 namespace {
 
-constexpr int NT = 1024;
+constexpr int NT = 512;   // 8 waves, 2 per SIMD: 256 registers each for the Q fragments and the accumulators
 constexpr int NWV = NT / 64;
 constexpr int QT = 16;   // query rows per workgroup
 constexpr int KT = 16;   // keys per tile
 
-template <int NF, int HPW>
+template <int NF, int HPW, int ROWS>
 __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __restrict__ out,
                                                                   const bf16_t* __restrict__ q,
                                                                   const bf16_t* __restrict__ k_cache,
@@ -37,15 +39,28 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
   float* P = lds;                    // [H][QT][KT] normalised weights of the current key tile
   float* PM = P + H * QT * KT;       // [H][QT][KT] mixed weights
   float* ST = PM + H * QT * KT;      // [H][QT][2]  (maximum, 1 / denominator)
+  float* TM = ST + 2 * H * QT;       // [H][H]      the mixing matrix
   __shared__ int s_pos[QT];
   const int seq = blockIdx.y;
-  const int q0 = a.q_starts[seq], q1 = a.q_starts[seq + 1];
-  const int row0 = q0 + QT * blockIdx.x;
-  if (row0 >= q1) return;
-  const int nr = min(QT, q1 - row0);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, grp = lane >> 4;
+  int row0, nr;
+  if constexpr (ROWS == 1) {   // a decode step: token `seq` is the one row of sequence `seq`
+    row0 = seq;
+    nr = 1;
+    if (a.slots[row0] < 0) {   // a padding row of the batch bucket
+      for (int i = tid; i < H * Dv; i += NT) out[(size_t)row0 * H * Dv + i] = 0;
+      return;
+    }
+  } else {
+    const int q0 = a.q_starts[seq], q1 = a.q_starts[seq + 1];
+    row0 = q0 + QT * blockIdx.x;
+    if (row0 >= q1) return;
+    nr = min(QT, q1 - row0);
+  }
   if (tid < QT) s_pos[tid] = tid < nr ? a.positions[row0 + tid] : -1;
+  if (a.mix != nullptr)
+    for (int i = tid; i < H * H; i += NT) TM[i] = a.mix[i];
   __syncthreads();
   const int p_last = s_pos[nr - 1];
   const int cs0 = a.chunk > 0 ? (s_pos[0] / a.chunk) * a.chunk : 0;
@@ -123,17 +138,23 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
   __syncthreads();
 
   // ---- pass 2 ----
-  // weights x values: this thread's head and its four consecutive value entries
+  constexpr int NDB = 2 * NF;   // 16-wide blocks of a head's values (Dv == D)
+  // ROWS == 16: out[16 rows x 16 values] blocks of this wave's heads on the fp32 matrix cores
+  f32x4 pacc[ROWS == QT ? HPW : 1][ROWS == QT ? NDB : 1];
+  // ROWS == 1 (a decode row): this thread's head and four consecutive value entries on the vector ALUs
+  // (H * Dv <= 4096 for every shape the launcher takes: at most MAXQ quads per thread)
+  constexpr int MAXQ = 2;
   const int nquads = (H * Dv) >> 2;
-  const bool has_quad = tid < nquads;
-  const int hq = has_quad ? (4 * tid) / Dv : 0, d0 = has_quad ? (4 * tid) % Dv : 0;
-  float acc[QT][4];
+  float acc1[MAXQ][4];
 #pragma unroll
-  for (int r = 0; r < QT; ++r) acc[r][0] = acc[r][1] = acc[r][2] = acc[r][3] = 0.f;
-  // mixing: this thread's (row, key) of the tile and its heads h0, h0 + 4, ...
-  const int rj = tid & (QT * KT - 1);
-  const int h0 = __builtin_amdgcn_readfirstlane(tid >> 8);
-  constexpr int HK = 16;   // heads per thread in the mixing: H <= 4 * HK
+  for (int qi = 0; qi < MAXQ; ++qi) acc1[qi][0] = acc1[qi][1] = acc1[qi][2] = acc1[qi][3] = 0.f;
+  if constexpr (ROWS == QT) {
+#pragma unroll
+    for (int u = 0; u < HPW; ++u)
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) pacc[u][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const int HB = (H + 15) >> 4;
 
   for (int jt = j_begin; jt <= p_last; jt += KT) {
 #pragma unroll
@@ -153,61 +174,109 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
     __syncthreads();
     const float* W = P;
     if (a.mix != nullptr) {
-      float s[HK];
+      if constexpr (ROWS == QT) {
+        // PM[h][rj] = sum_g mix[h][g] P[g][rj] as 16 x 16 blocks (16 heads x 16 of the tile's 256 (row, key)
+        // pairs) on mfma 16x16x4 f32: A = mix[h block][g .. g + 4], B = P[g .. g + 4][rj block]
+        for (int blk = wave; blk < HB * QT; blk += NWV) {
+          const int hb = blk / QT, rjb = blk % QT;
+          const int h = hb * 16 + col;
+          f32x4 c = {0.f, 0.f, 0.f, 0.f};
+          for (int g0 = 0; g0 < H; g0 += 4) {
+            const int g = g0 + grp;
+            const float av = (h < H && g < H) ? TM[h * H + g] : 0.f;
+            const float bv = g < H ? P[g * QT * KT + rjb * 16 + col] : 0.f;
+            c = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, c, 0, 0, 0);
+          }
 #pragma unroll
-      for (int k = 0; k < HK; ++k) s[k] = 0.f;
-      for (int g = 0; g < H; ++g) {
-        const float pv = P[g * QT * KT + rj];
-#pragma unroll
-        for (int k = 0; k < HK; ++k) {
-          const int h = h0 + 4 * k;
-          if (h < H) s[k] += a.mix[h * H + g] * pv;
+          for (int r = 0; r < 4; ++r) {
+            const int ho = hb * 16 + 4 * grp + r;
+            if (ho < H) PM[ho * QT * KT + rjb * 16 + col] = c[r];
+          }
         }
-      }
-#pragma unroll
-      for (int k = 0; k < HK; ++k) {
-        const int h = h0 + 4 * k;
-        if (h < H) PM[h * QT * KT + rj] = s[k];
+      } else {
+        for (int it = tid; it < H * KT; it += NT) {   // row 0 only
+          const int h = it / KT, j = it % KT;
+          float sm = 0.f;
+          for (int g = 0; g < H; ++g) sm += TM[h * H + g] * P[g * QT * KT + j];
+          PM[h * QT * KT + j] = sm;
+        }
       }
       __syncthreads();
       W = PM;
     }
-    if (has_quad) {
-      const float* wh = W + hq * QT * KT;
+    if constexpr (ROWS == QT) {
+      // out[row][d] += sum_key W[h][row][key] V[key][d]: A = W[h][row = col][4 k4 + grp], B = V[key][16 db + col]
+      size_t kbase[4];
 #pragma unroll
-      for (int j4 = 0; j4 < KT; j4 += 4) {
-        float v[4][4];
+      for (int k4 = 0; k4 < 4; ++k4) {
+        const int j = min(jt + 4 * k4 + grp, p_last);   // past the last row: weight 0, any valid value
+        kbase[k4] = ((size_t)bt[j / BS] * G * BS + j % BS) * Dv + col;
+      }
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          const int j = min(jt + j4 + jj, p_last);   // past the last row: weight 0, any valid value
-          const uint2 raw = *reinterpret_cast<const uint2*>(
-              v_cache + (((size_t)bt[j / BS] * G + hq / rep) * BS + j % BS) * Dv + d0);
-          v[jj][0] = lo_f(raw.x);
-          v[jj][1] = hi_f(raw.x);
-          v[jj][2] = lo_f(raw.y);
-          v[jj][3] = hi_f(raw.y);
+      for (int u = 0; u < HPW; ++u) {
+        const int h = wave + NWV * u;
+        if (h < H) {
+          const size_t hoff = (size_t)(h / rep) * BS * Dv;
+#pragma unroll
+          for (int k4 = 0; k4 < 4; ++k4) {
+            const float av = W[(h * QT + col) * KT + 4 * k4 + grp];
+            const bf16_t* vp = v_cache + kbase[k4] + hoff;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+              pacc[u][db] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bf2f(vp[16 * db]), pacc[u][db], 0, 0, 0);
+          }
         }
+      }
+    } else {
 #pragma unroll
-        for (int r = 0; r < QT; ++r) {
-          const f32x4 w4 = *reinterpret_cast<const f32x4*>(wh + r * KT + j4);
+      for (int qi = 0; qi < MAXQ; ++qi) {
+        const int quad = tid + qi * NT;
+        if (quad < nquads) {
+          const int hq = (4 * quad) / Dv, d0 = (4 * quad) % Dv;
+          const float* wh = W + hq * QT * KT;   // row 0
 #pragma unroll
-          for (int jj = 0; jj < 4; ++jj) {
+          for (int j4 = 0; j4 < KT; j4 += 4) {
+            const f32x4 w4 = *reinterpret_cast<const f32x4*>(wh + j4);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[r][e] += w4[jj] * v[jj][e];
+            for (int jj = 0; jj < 4; ++jj) {
+              const int j = min(jt + j4 + jj, p_last);
+              const uint2 raw = *reinterpret_cast<const uint2*>(
+                  v_cache + (((size_t)bt[j / BS] * G + hq / rep) * BS + j % BS) * Dv + d0);
+              acc1[qi][0] += w4[jj] * lo_f(raw.x);
+              acc1[qi][1] += w4[jj] * hi_f(raw.x);
+              acc1[qi][2] += w4[jj] * lo_f(raw.y);
+              acc1[qi][3] += w4[jj] * hi_f(raw.y);
+            }
           }
         }
       }
     }
     if (a.mix == nullptr) __syncthreads();   // P is rewritten by the next tile
   }
-  if (has_quad) {
+  if constexpr (ROWS == QT) {
 #pragma unroll
-    for (int r = 0; r < QT; ++r) {
-      if (r < nr) {
+    for (int u = 0; u < HPW; ++u) {
+      const int h = wave + NWV * u;
+      if (h < H) {
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int row = 4 * grp + r;
+            if (row < nr) out[(size_t)(row0 + row) * H * Dv + h * Dv + 16 * db + col] = f2bf(pacc[u][db][r]);
+          }
+        }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int qi = 0; qi < MAXQ; ++qi) {
+      const int quad = tid + qi * NT;
+      if (quad < nquads) {
         uint2 o;
-        o.x = pack2(acc[r][0], acc[r][1]);
-        o.y = pack2(acc[r][2], acc[r][3]);
-        *reinterpret_cast<uint2*>(out + (size_t)(row0 + r) * H * Dv + hq * Dv + d0) = o;
+        o.x = pack2(acc1[qi][0], acc1[qi][1]);
+        o.y = pack2(acc1[qi][2], acc1[qi][3]);
+        *reinterpret_cast<uint2*>(out + (size_t)row0 * H * Dv + 4 * quad) = o;
       }
     }
   }
@@ -216,7 +285,7 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
 template <int NF, int HPW>
 int launch(bf16_t* out, const bf16_t* q, const bf16_t* k, const bf16_t* v, const AttnArgs& a, int tiles, size_t lds,
            hipStream_t st) {
-  auto kern = chunk_attention_tile_kernel<NF, HPW>;
+  auto kern = a.q_starts == nullptr ? chunk_attention_tile_kernel<NF, HPW, 1> : chunk_attention_tile_kernel<NF, HPW, QT>;
   if (lds > 48 * 1024) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                              (int)lds);
@@ -232,7 +301,11 @@ int launch_nf(bf16_t* out, const bf16_t* q, const bf16_t* k, const bf16_t* v, co
   const int hpw = (a.H + NWV - 1) / NWV;
   if (hpw <= 1) return launch<NF, 1>(out, q, k, v, a, tiles, lds, st);
   if (hpw <= 2) return launch<NF, 2>(out, q, k, v, a, tiles, lds, st);
-  return launch<NF, 4>(out, q, k, v, a, tiles, lds, st);
+  if constexpr (NF <= 4) {
+    if (hpw <= 4) return launch<NF, 4>(out, q, k, v, a, tiles, lds, st);
+  }
+  if constexpr (NF <= 2) return launch<NF, 8>(out, q, k, v, a, tiles, lds, st);
+  return (int)hipErrorInvalidValue;
 }
 
 }  // namespace
@@ -240,24 +313,24 @@ int launch_nf(bf16_t* out, const bf16_t* q, const bf16_t* k, const bf16_t* v, co
 // 1 when ka_chunk_attention_tile takes the shape (see the head of this file)
 extern "C" int ka_chunk_attention_tile_ok(int H, int G, int D, int Dv, int BS) {
   const int nf = D / 32;
-  const int hpw = H <= NWV ? 1 : (H <= 2 * NWV ? 2 : 4);
-  const size_t lds = (size_t)(2 * H * QT * KT + 2 * H * QT) * sizeof(float);
-  return H > 0 && G > 0 && H % G == 0 && H <= 64 && D % 32 == 0 && (nf <= 4 || nf == 6 || nf == 8) && hpw * nf <= 8 &&
-         Dv % 4 == 0 &&
-         H * Dv <= 4 * NT && BS > 0 && lds <= 150 * 1024;
+  const int hpw = H <= NWV ? 1 : (H <= 2 * NWV ? 2 : (H <= 4 * NWV ? 4 : 8));
+  const size_t lds = (size_t)(2 * H * QT * KT + 2 * H * QT + H * H) * sizeof(float);
+  return H > 0 && G > 0 && H % G == 0 && H <= 64 && D % 32 == 0 && (nf <= 4 || nf == 6 || nf == 8) && hpw * nf <= 16 &&
+         Dv == D && BS > 0 && lds <= 150 * 1024;
 }
 
-// max_q: the longest run of rows of one sequence in this step (the grid's x extent is ceil(max_q / 16))
+// max_q: the longest run of rows of one sequence in this step (the grid's x extent is ceil(max_q / 16)).
+// q_starts null: a decode step, token t is the single row of block-table row t (one workgroup per token).
 extern "C" int ka_chunk_attention_tile(void* out, const void* q, const void* k_cache, const void* v_cache,
                                        const int* block_tables, const int* q_starts, int num_seqs, const int* positions,
                                        const int* slots, const float* mix, int max_q, int H, int G, int D, int Dv,
                                        int chunk, int BS, int max_blocks, int sink, float scale, float cap,
                                        hipStream_t st) {
   if (num_seqs <= 0 || max_q <= 0) return 0;
-  if (!ka_chunk_attention_tile_ok(H, G, D, Dv, BS) || q_starts == nullptr || chunk < 0) return (int)hipErrorInvalidValue;
+  if (!ka_chunk_attention_tile_ok(H, G, D, Dv, BS) || chunk < 0) return (int)hipErrorInvalidValue;
   AttnArgs a{block_tables, q_starts, num_seqs, positions, slots, mix, H, G, D, Dv, chunk, BS, max_blocks, sink, scale, cap};
-  const size_t lds = (size_t)(2 * H * QT * KT + 2 * H * QT) * sizeof(float);
-  const int tiles = (max_q + QT - 1) / QT;
+  const size_t lds = (size_t)(2 * H * QT * KT + 2 * H * QT + H * H) * sizeof(float);
+  const int tiles = q_starts == nullptr ? 1 : (max_q + QT - 1) / QT;
   bf16_t* o = (bf16_t*)out;
   const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k_cache, *vv = (const bf16_t*)v_cache;
   switch (D / 32) {

@@ -133,14 +133,16 @@ def chunk_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     assert q_starts is None or (q_starts.dtype == torch.int32 and q_starts.shape[0] == block_tables.shape[0] + 1)
     assert q_starts is not None or block_tables.shape[0] >= T
     assert mix is None or (mix.dtype == torch.float32 and mix.shape == (H, H) and mix.is_contiguous())
-    if (q_starts is not None and max_q >= TILE_MIN_Q and q.dtype == torch.bfloat16
+    if ((q_starts is None or max_q >= TILE_MIN_Q) and q.dtype == torch.bfloat16
             and lib.ka_chunk_attention_tile_ok(H, G, D, Dv, BS)):
-        # rows past the last sequence (a padded step) belong to no tile: they stay zero
-        out = torch.zeros((T, H * Dv), dtype=q.dtype, device=q.device)
+        # varlen: rows past the last sequence (a padded step) belong to no tile and stay zero;
+        # decode (q_starts None): one workgroup per token writes every row
+        varlen = q_starts is not None
+        out = (torch.zeros if varlen else torch.empty)((T, H * Dv), dtype=q.dtype, device=q.device)
         check(lib.ka_chunk_attention_tile(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(q_starts),
-                                          block_tables.shape[0], _p(positions), _p(slots), _p(mix), int(max_q), H, G, D,
-                                          Dv, int(chunk), BS, block_tables.shape[1], int(bool(sink)), float(scale),
-                                          float(cap), _stream()), "chunk_attention_tile")
+                                          block_tables.shape[0] if varlen else T, _p(positions), _p(slots), _p(mix),
+                                          int(max_q) if varlen else 1, H, G, D, Dv, int(chunk), BS, block_tables.shape[1],
+                                          int(bool(sink)), float(scale), float(cap), _stream()), "chunk_attention_tile")
         return out
     out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
     check(lib.ka_chunk_attention(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(q_starts),

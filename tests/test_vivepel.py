@@ -263,6 +263,9 @@ def test_chunk_attention_tile_kernel(H, G, D, chunk, cap, sink, mixed):
         # the per-token kernel on the same inputs agrees too (max_q 0 keeps it off the tile kernel)
         got1, _ = _attention_case("cuda", H, G, D, chunk, cap, sink, mix, list(range(lo, n)), n, dtype=torch.bfloat16, seed=lo)
         assert torch.allclose(got, got1, rtol=2e-2, atol=2e-2)
+    for p in (0, 1, 15, 16, 17, 47, 48, 89):         # one decoded row per workgroup on the same kernel
+        got, want = _attention_case("cuda", H, G, D, chunk, cap, sink, mix, [p], 90, dtype=torch.bfloat16, seed=p)
+        assert torch.allclose(got, want, rtol=2e-2, atol=2e-2), (p, float((got - want).abs().max()))
 
 
 @pytest.mark.parametrize("device", DEVICES)
