@@ -9,11 +9,10 @@
 //              token-major pages (lane = key, 8 consecutive head entries), no LDS staging;
 //   pass 1     per head and row, the running maximum and denominator over the row's visible keys
 //              (soft cap, chunk mask, sink), kept in LDS as (maximum, 1 / denominator);
-//   pass 2     per tile of 16 keys: the normalised fp32 weights of all heads go to LDS, are mixed over
-//              the heads, and multiplied with the values, both on the fp32 matrix instruction
-//              (mfma 16x16x4 f32): the weights are never rounded to bf16, the bf16 values are widened.
-// Only Q K^T runs at the bf16 MFMA rate, where bf16 inputs lose nothing; everything that the design
-// wants in 32 bits runs at the fp32 matrix rate (1/16 of the bf16 rate), which is this kernel's roofline.
+//   pass 2     per tile of 16 keys: the normalised fp32 weights of all heads go to LDS and are mixed over
+//              the heads on the fp32 matrix instruction (mfma 16x16x4 f32); weights x values runs on
+//              mfma 16x16x16 bf16 with each fp32 weight split exactly into three bf16 terms
+//              (hi + mid + lo = the fp32 value), so no weight is rounded and the sums stay fp32.
 // A decode step (q_starts null) runs the same kernel with one row per workgroup: scores on MFMA with
 // one useful row, mixing and weights x values for that row on the vector ALUs.
 //
@@ -27,6 +26,31 @@ constexpr int NT = 512;   // 8 waves, 2 per SIMD: 256 registers each for the Q f
 constexpr int NWV = NT / 64;
 constexpr int QT = 16;   // query rows per workgroup
 constexpr int KT = 16;   // keys per tile
+constexpr int MAXPG = 4096;   // staged block-table entries (the launcher checks max_blocks against it)
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+// exp and tanh through the hardware exponential (v_exp_f32, about 1 ulp): this kernel serves the bf16
+// engine; the fp32 engine's attention (attention_chunk.hip) keeps the library functions
+KA_DEV float fast_tanh(float y) {
+  y = fminf(fmaxf(y, -15.f), 15.f);
+  const float e = __expf(2.f * y);
+  return (e - 1.f) * __frcp_rn(e + 1.f);
+}
+
+// p = hi + mid + lo exactly, each term a bf16: an fp32 weight as three bf16 MFMA operands
+KA_DEV void split3(const f32x4& p, s16x4& hi, s16x4& mid, s16x4& lo) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const bf16_t h = f2bf(p[i]);
+    const float r1 = p[i] - bf2f(h);
+    const bf16_t m = f2bf(r1);
+    const float r2 = r1 - bf2f(m);
+    hi[i] = (short)h;
+    mid[i] = (short)m;
+    lo[i] = (short)f2bf(r2);
+  }
+}
 
 template <int NF, int HPW, int ROWS>
 __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __restrict__ out,
@@ -40,6 +64,7 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
   float* PM = P + H * QT * KT;       // [H][QT][KT] mixed weights
   float* ST = PM + H * QT * KT;      // [H][QT][2]  (maximum, 1 / denominator)
   float* TM = ST + 2 * H * QT;       // [H][H]      the mixing matrix
+  int* PG = reinterpret_cast<int*>(TM + H * H);   // [max_blocks] pages of the keys this workgroup visits
   __shared__ int s_pos[QT];
   const int seq = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -65,8 +90,17 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
   const int p_last = s_pos[nr - 1];
   const int cs0 = a.chunk > 0 ? (s_pos[0] / a.chunk) * a.chunk : 0;
   const int j_begin = cs0 & ~(KT - 1);
-  const int* bt = a.block_tables + (size_t)seq * a.max_blocks;
   const int rep = H / G;
+  // the pages of keys j_begin .. p_last, staged once: every later page lookup is an LDS read instead of
+  // a global load in front of the key / value loads that depend on it
+  const int pg0 = j_begin / BS;
+  {
+    const int* btg = a.block_tables + (size_t)seq * a.max_blocks;
+    const int npg = p_last / BS - pg0 + 1;
+    for (int i = tid; i < npg; i += NT) PG[i] = btg[pg0 + i];   // npg <= max_blocks, which sized PG
+  }
+  __syncthreads();
+  const int* bt = PG - pg0;   // bt[j / BS] as before
   // the four S rows of this lane: row = 4 * grp + r; visible keys lo[r] .. hi[r] (hi < lo: no row)
   int lo[4], hi[4];
 #pragma unroll
@@ -87,10 +121,16 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
     }
   }
 
+  const float inv_cap = a.cap > 0.f ? 1.0f / a.cap : 0.f;
   // soft-capped, masked scores of head g (slot u) against the key tile at jt: x[r] for row 4 grp + r, key jt + col
-  auto scores = [&](int u, int g, int jt, float (&x)[4]) {
-    const int j = min(jt + col, p_last);      // keys past the tile's last row: a valid address, masked below
-    const bf16_t* kp = k_cache + (((size_t)bt[j / BS] * G + g / rep) * BS + j % BS) * D + 8 * grp;
+  // kbase_of(jt): this lane's key row of the tile (head 0) in the cache; keys past the tile's last row
+  // take a valid address and are masked in `scores`
+  auto kbase_of = [&](int jt) -> size_t {
+    const int j = min(jt + col, p_last);
+    return ((size_t)bt[j / BS] * G * BS + j % BS) * D + 8 * grp;
+  };
+  auto scores = [&](int u, int g, int jt, size_t kb, float (&x)[4]) {
+    const bf16_t* kp = k_cache + kb + (size_t)(g / rep) * BS * D;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < NF; ++ks)
@@ -99,7 +139,7 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       float s = acc[r] * a.scale;
-      if (a.cap > 0.f) s = a.cap * tanhf(s / a.cap);
+      if (a.cap > 0.f) s = a.cap * fast_tanh(s * inv_cap);
       x[r] = (jj <= hi[r] && jj >= lo[r]) ? s : -INFINITY;
     }
   };
@@ -117,12 +157,12 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
       }
       for (int jt = j_begin; jt <= p_last; jt += KT) {
         float x[4];
-        scores(u, g, jt, x);
+        scores(u, g, jt, kbase_of(jt), x);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float mn = fmaxf(m[r], row16_max(x[r]));
-          const float e = row16_sum(x[r] == -INFINITY ? 0.f : expf(x[r] - mn));
-          l[r] = l[r] * (m[r] == -INFINITY ? 0.f : expf(m[r] - mn)) + e;
+          const float e = row16_sum(x[r] == -INFINITY ? 0.f : __expf(x[r] - mn));
+          l[r] = l[r] * (m[r] == -INFINITY ? 0.f : __expf(m[r] - mn)) + e;
           m[r] = mn;
         }
       }
@@ -157,16 +197,17 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
   const int HB = (H + 15) >> 4;
 
   for (int jt = j_begin; jt <= p_last; jt += KT) {
+    const size_t kb = kbase_of(jt);
 #pragma unroll
     for (int u = 0; u < HPW; ++u) {
       const int g = wave + NWV * u;
       if (g < H) {
         float x[4];
-        scores(u, g, jt, x);
+        scores(u, g, jt, kb, x);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int row = 4 * grp + r;
-          const float w = x[r] == -INFINITY ? 0.f : expf(x[r] - ST[(g * QT + row) * 2]) * ST[(g * QT + row) * 2 + 1];
+          const float w = x[r] == -INFINITY ? 0.f : __expf(x[r] - ST[(g * QT + row) * 2]) * ST[(g * QT + row) * 2 + 1];
           P[(g * QT + row) * KT + col] = w;
         }
       }
@@ -205,25 +246,30 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
       W = PM;
     }
     if constexpr (ROWS == QT) {
-      // out[row][d] += sum_key W[h][row][key] V[key][d]: A = W[h][row = col][4 k4 + grp], B = V[key][16 db + col]
+      // out[row][d] += sum_key W[h][row][key] V[key][d] on mfma 16x16x16 bf16, three times: the fp32
+      // weight is split exactly into three bf16 terms (split3), the values are bf16 already.
+      // A = W[h][row = col][4 grp .. + 4], B = V[key 4 grp .. + 4][16 db + col]
       size_t kbase[4];
 #pragma unroll
-      for (int k4 = 0; k4 < 4; ++k4) {
-        const int j = min(jt + 4 * k4 + grp, p_last);   // past the last row: weight 0, any valid value
-        kbase[k4] = ((size_t)bt[j / BS] * G * BS + j % BS) * Dv + col;
+      for (int i = 0; i < 4; ++i) {
+        const int j = min(jt + 4 * grp + i, p_last);   // past the last row: weight 0, any valid value
+        kbase[i] = ((size_t)bt[j / BS] * G * BS + j % BS) * Dv + col;
       }
 #pragma unroll
       for (int u = 0; u < HPW; ++u) {
         const int h = wave + NWV * u;
         if (h < H) {
           const size_t hoff = (size_t)(h / rep) * BS * Dv;
+          s16x4 ahi, amid, alo;
+          split3(*reinterpret_cast<const f32x4*>(W + (h * QT + col) * KT + 4 * grp), ahi, amid, alo);
 #pragma unroll
-          for (int k4 = 0; k4 < 4; ++k4) {
-            const float av = W[(h * QT + col) * KT + 4 * k4 + grp];
-            const bf16_t* vp = v_cache + kbase[k4] + hoff;
+          for (int db = 0; db < NDB; ++db) {
+            s16x4 b;
 #pragma unroll
-            for (int db = 0; db < NDB; ++db)
-              pacc[u][db] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bf2f(vp[16 * db]), pacc[u][db], 0, 0, 0);
+            for (int i = 0; i < 4; ++i) b[i] = (short)v_cache[kbase[i] + hoff + 16 * db];
+            pacc[u][db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ahi, b, pacc[u][db], 0, 0, 0);
+            pacc[u][db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(amid, b, pacc[u][db], 0, 0, 0);
+            pacc[u][db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(alo, b, pacc[u][db], 0, 0, 0);
           }
         }
       }
@@ -314,7 +360,7 @@ int launch_nf(bf16_t* out, const bf16_t* q, const bf16_t* k, const bf16_t* v, co
 extern "C" int ka_chunk_attention_tile_ok(int H, int G, int D, int Dv, int BS) {
   const int nf = D / 32;
   const int hpw = H <= NWV ? 1 : (H <= 2 * NWV ? 2 : (H <= 4 * NWV ? 4 : 8));
-  const size_t lds = (size_t)(2 * H * QT * KT + 2 * H * QT + H * H) * sizeof(float);
+  const size_t lds = (size_t)(2 * H * QT * KT + 2 * H * QT + H * H) * sizeof(float);   // + the staged pages
   return H > 0 && G > 0 && H % G == 0 && H <= 64 && D % 32 == 0 && (nf <= 4 || nf == 6 || nf == 8) && hpw * nf <= 16 &&
          Dv == D && BS > 0 && lds <= 150 * 1024;
 }
@@ -329,7 +375,8 @@ extern "C" int ka_chunk_attention_tile(void* out, const void* q, const void* k_c
   if (num_seqs <= 0 || max_q <= 0) return 0;
   if (!ka_chunk_attention_tile_ok(H, G, D, Dv, BS) || chunk < 0) return (int)hipErrorInvalidValue;
   AttnArgs a{block_tables, q_starts, num_seqs, positions, slots, mix, H, G, D, Dv, chunk, BS, max_blocks, sink, scale, cap};
-  const size_t lds = (size_t)(2 * H * QT * KT + 2 * H * QT + H * H) * sizeof(float);
+  if (max_blocks > MAXPG) return (int)hipErrorInvalidValue;
+  const size_t lds = (size_t)(2 * H * QT * KT + 2 * H * QT + H * H + max_blocks) * sizeof(float);
   const int tiles = q_starts == nullptr ? 1 : (max_q + QT - 1) / QT;
   bf16_t* o = (bf16_t*)out;
   const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k_cache, *vv = (const bf16_t*)v_cache;

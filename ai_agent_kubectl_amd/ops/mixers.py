@@ -17,6 +17,7 @@ from . import reference as ref
 from ._hip import check, require_mixers
 
 
+TILE_MAX_BLOCKS = 4096   # block-table width the tile kernel stages in LDS (csrc/attention_chunk_tile.hip MAXPG)
 TILE_MIN_Q = 8   # varlen steps whose longest row run is shorter stay on the per-token attention kernel
 
 
@@ -134,7 +135,7 @@ def chunk_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     assert q_starts is not None or block_tables.shape[0] >= T
     assert mix is None or (mix.dtype == torch.float32 and mix.shape == (H, H) and mix.is_contiguous())
     if ((q_starts is None or max_q >= TILE_MIN_Q) and q.dtype == torch.bfloat16
-            and lib.ka_chunk_attention_tile_ok(H, G, D, Dv, BS)):
+            and block_tables.shape[1] <= TILE_MAX_BLOCKS and lib.ka_chunk_attention_tile_ok(H, G, D, Dv, BS)):
         # varlen: rows past the last sequence (a padded step) belong to no tile and stay zero;
         # decode (q_starts None): one workgroup per token writes every row
         varlen = q_starts is not None
