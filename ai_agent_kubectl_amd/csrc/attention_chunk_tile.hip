@@ -22,10 +22,11 @@
 
 namespace {
 
-constexpr int NT = 512;   // 8 waves, 2 per SIMD: 256 registers each for the Q fragments and the accumulators
+constexpr int NT = 1024;   // 16 waves, 4 per SIMD
 constexpr int NWV = NT / 64;
 constexpr int QT = 16;   // query rows per workgroup
 constexpr int KT = 16;   // keys per tile
+constexpr int VST = 20;        // keys per value entry in the staged value tile (16 + padding, 8-byte aligned rows)
 constexpr int MAXPG = 4096;   // staged block-table entries (the launcher checks max_blocks against it)
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -65,6 +66,9 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
   float* ST = PM + H * QT * KT;      // [H][QT][2]  (maximum, 1 / denominator)
   float* TM = ST + 2 * H * QT;       // [H][H]      the mixing matrix
   int* PG = reinterpret_cast<int*>(TM + H * H);   // [max_blocks] pages of the keys this workgroup visits
+  // [G][Dv][VST] the key tile's values, entry-major (16 keys of one value entry side by side): the B
+  // operand of weights x values is then one 8-byte LDS read; filled from 16-byte global loads
+  bf16_t* VS = reinterpret_cast<bf16_t*>(PG + a.max_blocks);
   __shared__ int s_pos[QT];
   const int seq = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -93,10 +97,11 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
   const int rep = H / G;
   // the pages of keys j_begin .. p_last, staged once: every later page lookup is an LDS read instead of
   // a global load in front of the key / value loads that depend on it
-  const int pg0 = j_begin / BS;
+  const int bs_sh = __builtin_ctz(BS);   // the page size is a power of two (the launcher checks)
+  const int pg0 = j_begin >> bs_sh;
   {
     const int* btg = a.block_tables + (size_t)seq * a.max_blocks;
-    const int npg = p_last / BS - pg0 + 1;
+    const int npg = (p_last >> bs_sh) - pg0 + 1;
     for (int i = tid; i < npg; i += NT) PG[i] = btg[pg0 + i];   // npg <= max_blocks, which sized PG
   }
   __syncthreads();
@@ -127,7 +132,7 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
   // take a valid address and are masked in `scores`
   auto kbase_of = [&](int jt) -> size_t {
     const int j = min(jt + col, p_last);
-    return ((size_t)bt[j / BS] * G * BS + j % BS) * D + 8 * grp;
+    return ((size_t)bt[j >> bs_sh] * G * BS + (j & (BS - 1))) * D + 8 * grp;
   };
   auto scores = [&](int u, int g, int jt, size_t kb, float (&x)[4]) {
     const bf16_t* kp = k_cache + kb + (size_t)(g / rep) * BS * D;
@@ -183,7 +188,7 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
   f32x4 pacc[ROWS == QT ? HPW : 1][ROWS == QT ? NDB : 1];
   // ROWS == 1 (a decode row): this thread's head and four consecutive value entries on the vector ALUs
   // (H * Dv <= 4096 for every shape the launcher takes: at most MAXQ quads per thread)
-  constexpr int MAXQ = 2;
+  constexpr int MAXQ = 1;
   const int nquads = (H * Dv) >> 2;
   float acc1[MAXQ][4];
 #pragma unroll
@@ -213,6 +218,23 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
       }
     }
     __syncthreads();
+    if constexpr (ROWS == QT) {
+      // stage the tile's values (every workgroup-mate is past the previous tile's reads of VS here)
+      const int c8 = Dv >> 3;
+      for (int it = tid; it < G * KT * c8; it += NT) {
+        const int d8 = it % c8, key = (it / c8) % KT, c = it / (c8 * KT);
+        const int j = min(jt + key, p_last);
+        const uint4 raw = *reinterpret_cast<const uint4*>(
+            v_cache + (((size_t)bt[j >> bs_sh] * G + c) * BS + (j & (BS - 1))) * Dv + 8 * d8);
+        bf16_t* dst = VS + ((size_t)(c * Dv + 8 * d8)) * VST + key;
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          dst[(2 * i) * VST] = (bf16_t)(w[i] & 0xffffu);
+          dst[(2 * i + 1) * VST] = (bf16_t)(w[i] >> 16);
+        }
+      }
+    }
     const float* W = P;
     if (a.mix != nullptr) {
       if constexpr (ROWS == QT) {
@@ -244,29 +266,23 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
       }
       __syncthreads();
       W = PM;
+    } else if (ROWS == QT) {
+      __syncthreads();   // the staged values are read below
     }
     if constexpr (ROWS == QT) {
       // out[row][d] += sum_key W[h][row][key] V[key][d] on mfma 16x16x16 bf16, three times: the fp32
       // weight is split exactly into three bf16 terms (split3), the values are bf16 already.
       // A = W[h][row = col][4 grp .. + 4], B = V[key 4 grp .. + 4][16 db + col]
-      size_t kbase[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int j = min(jt + 4 * grp + i, p_last);   // past the last row: weight 0, any valid value
-        kbase[i] = ((size_t)bt[j / BS] * G * BS + j % BS) * Dv + col;
-      }
 #pragma unroll
       for (int u = 0; u < HPW; ++u) {
         const int h = wave + NWV * u;
         if (h < H) {
-          const size_t hoff = (size_t)(h / rep) * BS * Dv;
           s16x4 ahi, amid, alo;
           split3(*reinterpret_cast<const f32x4*>(W + (h * QT + col) * KT + 4 * grp), ahi, amid, alo);
+          const bf16_t* vs = VS + ((size_t)((h / rep) * Dv + col)) * VST + 4 * grp;
 #pragma unroll
           for (int db = 0; db < NDB; ++db) {
-            s16x4 b;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) b[i] = (short)v_cache[kbase[i] + hoff + 16 * db];
+            const s16x4 b = *reinterpret_cast<const s16x4*>(vs + 16 * db * VST);
             pacc[u][db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ahi, b, pacc[u][db], 0, 0, 0);
             pacc[u][db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(amid, b, pacc[u][db], 0, 0, 0);
             pacc[u][db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(alo, b, pacc[u][db], 0, 0, 0);
@@ -287,7 +303,7 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
             for (int jj = 0; jj < 4; ++jj) {
               const int j = min(jt + j4 + jj, p_last);
               const uint2 raw = *reinterpret_cast<const uint2*>(
-                  v_cache + (((size_t)bt[j / BS] * G + hq / rep) * BS + j % BS) * Dv + d0);
+                  v_cache + (((size_t)bt[j >> bs_sh] * G + hq / rep) * BS + (j & (BS - 1))) * Dv + d0);
               acc1[qi][0] += w4[jj] * lo_f(raw.x);
               acc1[qi][1] += w4[jj] * hi_f(raw.x);
               acc1[qi][2] += w4[jj] * lo_f(raw.y);
@@ -347,10 +363,7 @@ int launch_nf(bf16_t* out, const bf16_t* q, const bf16_t* k, const bf16_t* v, co
   const int hpw = (a.H + NWV - 1) / NWV;
   if (hpw <= 1) return launch<NF, 1>(out, q, k, v, a, tiles, lds, st);
   if (hpw <= 2) return launch<NF, 2>(out, q, k, v, a, tiles, lds, st);
-  if constexpr (NF <= 4) {
-    if (hpw <= 4) return launch<NF, 4>(out, q, k, v, a, tiles, lds, st);
-  }
-  if constexpr (NF <= 2) return launch<NF, 8>(out, q, k, v, a, tiles, lds, st);
+  if constexpr (NF <= 2) return launch<NF, 4>(out, q, k, v, a, tiles, lds, st);
   return (int)hipErrorInvalidValue;
 }
 
@@ -359,10 +372,10 @@ int launch_nf(bf16_t* out, const bf16_t* q, const bf16_t* k, const bf16_t* v, co
 // 1 when ka_chunk_attention_tile takes the shape (see the head of this file)
 extern "C" int ka_chunk_attention_tile_ok(int H, int G, int D, int Dv, int BS) {
   const int nf = D / 32;
-  const int hpw = H <= NWV ? 1 : (H <= 2 * NWV ? 2 : (H <= 4 * NWV ? 4 : 8));
-  const size_t lds = (size_t)(2 * H * QT * KT + 2 * H * QT + H * H) * sizeof(float);   // + the staged pages
-  return H > 0 && G > 0 && H % G == 0 && H <= 64 && D % 32 == 0 && (nf <= 4 || nf == 6 || nf == 8) && hpw * nf <= 16 &&
-         Dv == D && BS > 0 && lds <= 150 * 1024;
+  const int hpw = H <= NWV ? 1 : (H <= 2 * NWV ? 2 : 4);
+  const size_t lds = (size_t)(2 * H * QT * KT + 2 * H * QT + H * H) * sizeof(float) + (size_t)G * Dv * VST * 2;   // + the staged pages
+  return H > 0 && G > 0 && H % G == 0 && H <= 64 && D % 32 == 0 && (nf <= 4 || nf == 6 || nf == 8) && hpw * nf <= 8 &&
+         Dv == D && (BS & (BS - 1)) == 0 && BS > 0 && lds <= 140 * 1024;
 }
 
 // max_q: the longest run of rows of one sequence in this step (the grid's x extent is ceil(max_q / 16)).
@@ -376,7 +389,7 @@ extern "C" int ka_chunk_attention_tile(void* out, const void* q, const void* k_c
   if (!ka_chunk_attention_tile_ok(H, G, D, Dv, BS) || chunk < 0) return (int)hipErrorInvalidValue;
   AttnArgs a{block_tables, q_starts, num_seqs, positions, slots, mix, H, G, D, Dv, chunk, BS, max_blocks, sink, scale, cap};
   if (max_blocks > MAXPG) return (int)hipErrorInvalidValue;
-  const size_t lds = (size_t)(2 * H * QT * KT + 2 * H * QT + H * H + max_blocks) * sizeof(float);
+  const size_t lds = (size_t)(2 * H * QT * KT + 2 * H * QT + H * H + max_blocks) * sizeof(float) + (size_t)G * Dv * VST * 2;
   const int tiles = q_starts == nullptr ? 1 : (max_q + QT - 1) / QT;
   bf16_t* o = (bf16_t*)out;
   const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k_cache, *vv = (const bf16_t*)v_cache;

@@ -65,8 +65,13 @@ def build_engine(opts: EngineOptions, comm=None, metrics=None) -> LLMEngine:
     tok = get_tokenizer(cfg.vocab_size, cfg.tokenizer, tokenizer_path(opts.weights))
     dev = torch.device(opts.device)
     if dev.type == "cuda":
-        from ..ops._hip import require
-        require()  # fail loudly: the GPU path never runs without the HIP kernels
+        # fail loudly: the GPU path never runs without the HIP kernels of the model's family
+        if getattr(cfg, "family", "llama") == "vivepel":
+            from ..ops._hip import require_mixers
+            require_mixers()
+        else:
+            from ..ops._hip import require
+            require()
         torch.cuda.set_device(dev.index if dev.index is not None else torch.cuda.current_device())
     if opts.dtype not in ("bfloat16", "float32"):
         raise ValueError(f"dtype {opts.dtype!r}: bfloat16 or float32")
@@ -115,9 +120,6 @@ def build_engine(opts: EngineOptions, comm=None, metrics=None) -> LLMEngine:
     else:
         want = opts.kv_cache_tokens // opts.block_size if opts.kv_cache_tokens > 0 else 4096
         num_blocks = min(max(want, min_blocks), 4096)
-    if dev.type == "cuda" and family == "vivepel":
-        from ..ops._hip import require_mixers
-        require_mixers()
     masks = build_masks(tok, allow_eos=not opts.ignore_eos) if opts.safe_decode else None
     if comm is not None and opts.tp_size > 1:
         from ..parallel.custom_allreduce import maybe_enable
