@@ -105,8 +105,10 @@ class Settings:
 
     # --- LLM backend selection ---
     LLM_BACKEND: str = "stub"            # stub | engine | openai
-    MODEL: str = "llama3-8b"             # llama3-8b | llama3-70b | mixtral-8x7b | tiny-llama | tiny-mixtral
-    WEIGHTS: str = "random:0"            # safetensors dir/file or random:<seed>
+    MODEL: str = "llama3-8b"             # a preset (llama3-8b | llama3-70b | mixtral-8x7b | vivepel-8b | tiny-*) or a
+                                         # checkpoint folder (config.json names the architecture, e.g. Vivepel)
+    WEIGHTS: str = "random:0"            # safetensors dir/file or random:<seed> (a MODEL folder brings its own)
+    DTYPE: str = "bfloat16"              # bfloat16 | float32 (float32: the fp32-residual families only, e.g. Vivepel)
     TP: int = 1
     DP: int = 1
     ENGINE_PROCESS: bool = True          # run the engine (a TP group) in its own process(es): the API keeps its GIL

@@ -30,7 +30,7 @@ constexpr int NW = NT / 64;
 constexpr int KT = 64;        // keys per tile
 constexpr int MAX_HEADS = 64;
 static_assert(KT == 64, "pass 1 reads one key of the tile per lane");
-constexpr int MAX_ACC = 16;   // output values per thread: H * Dv <= NT * MAX_ACC
+constexpr int MAX_ACC = 32;   // output values per thread: H * Dv <= NT * MAX_ACC
 constexpr int MAX_DL = 8;     // head entries per lane: D <= 64 * MAX_DL
 
 template <typename T>
@@ -290,8 +290,14 @@ extern "C" int ka_chunk_attention(void* out, const void* q, const void* k_cache,
   if (H <= 0 || G <= 0 || H % G || H > MAX_HEADS || H * Dv > NT * MAX_ACC || D <= 0 || Dv <= 0 || BS <= 0 || chunk < 0)
     return (int)hipErrorInvalidValue;
   const size_t lds = (size_t)(H * D + 2 * H * KT + 2 * H) * sizeof(float);
-  if (lds > 60 * 1024) return (int)hipErrorInvalidValue;
+  if (lds > 150 * 1024) return (int)hipErrorInvalidValue;
   AttnArgs a{block_tables, q_starts, num_seqs, positions, slots, mix, H, G, D, Dv, chunk, BS, max_blocks, sink, scale, cap};
+  if (lds > 48 * 1024) {   // wide models: more dynamic LDS than the default limit
+    const void* fn = f32 ? reinterpret_cast<const void*>(chunk_attention_kernel<float>)
+                         : reinterpret_cast<const void*>(chunk_attention_kernel<bf16_t>);
+    const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+  }
   if (f32)
     chunk_attention_kernel<float><<<T, NT, lds, st>>>((float*)out, (const float*)q, (const float*)k_cache,
                                                       (const float*)v_cache, a);

@@ -55,7 +55,7 @@ class EngineOptions:
                    graph_buckets=tuple(b for b in s.graph_buckets() if b <= s.MAX_BATCH) or (1,),
                    safe_decode=s.SAFE_DECODE, ignore_eos=s.IGNORE_EOS, prefix_caching=s.PREFIX_CACHING,
                    kv_cache_tokens=int(os.environ.get("KV_CACHE_TOKENS", 0)),
-                   max_model_len=int(os.environ.get("MAX_MODEL_LEN", 8192)),
+                   max_model_len=int(os.environ.get("MAX_MODEL_LEN", 8192)), dtype=getattr(s, "DTYPE", "bfloat16"),
                    device="cuda" if torch.cuda.is_available() else "cpu")
 
 

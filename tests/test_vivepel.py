@@ -268,6 +268,20 @@ def test_chunk_attention_tile_kernel(H, G, D, chunk, cap, sink, mixed):
         assert torch.allclose(got, want, rtol=2e-2, atol=2e-2), (p, float((got - want).abs().max()))
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_wide_model_attention(dtype):
+    """64 heads of 128: more LDS and more accumulators than the small shapes use (the kernel with one
+    workgroup per token; the tile kernel does not take this width)."""
+    H, G, D = 64, 8, 128
+    mix = torch.eye(H) * 0.6 + torch.randn(H, H, generator=torch.Generator().manual_seed(9)) * 0.05
+    t = 1e-4 if dtype == torch.float32 else 2e-2
+    got, want = _attention_case("cuda", H, G, D, 32, 30.0, True, mix, list(range(30, 36)), 36, dtype=dtype, max_q=6)
+    assert torch.allclose(got, want, rtol=t, atol=t)
+    got, want = _attention_case("cuda", H, G, D, 32, 30.0, True, mix, [35], 36, dtype=dtype)
+    assert torch.allclose(got, want, rtol=t, atol=t)
+
+
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("decode", [False, True])
 def test_chunk_edges_one_score_stands_out(device, decode):
@@ -436,6 +450,32 @@ def test_generate_greedy_through_scheduler(tmp_path, device):
         for _ in range(10):
             toks.append(int(want_logits(config, W, toks)[-1].argmax()))
         assert s.generated == toks[len(p):]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_steps_that_want_nothing(tmp_path, device):
+    """Portions whose logits nobody asks for (and a request that is ended right after its portion)
+    still fill the cache; later positions match."""
+    config = variant("base")
+    W = oracle.random_weights(config, seed=22)
+    sess = session(write_checkpoint(tmp_path / "m", config, W), device)
+    toks = tokens_for(config, 30, seed=10)
+    assert sess.step([{"id": "x", "tokens": toks[:11], "want": []}], []).shape == (0, config["vocab"])
+    assert sess.step([{"id": "x", "tokens": toks[11:12], "want": []}, {"id": "y", "tokens": toks[:3], "want": []}],
+                     ["y"]).shape[0] == 0
+    got = sess.step([{"id": "x", "tokens": toks[12:], "want": [0, 17]}], ["x"])
+    want = want_logits(config, W, toks)
+    assert rel_err(got, want[[12, 29]]) < tol("float32")
+    assert sess.engine.bm.num_free == sess.engine.bm.num_blocks
+
+
+def test_settings_select_a_checkpoint_folder_and_dtype(tmp_path):
+    from ai_agent_kubectl_amd.config import Settings
+    from ai_agent_kubectl_amd.engine.builder import EngineOptions
+
+    path = write_checkpoint(tmp_path / "m", variant("base"), oracle.random_weights(variant("base"), seed=1))
+    opts = EngineOptions.from_settings(Settings(MODEL=path, DTYPE="float32"))
+    assert opts.model == path and opts.dtype == "float32"
 
 
 def test_config_reader_rejects_what_it_does_not_know(tmp_path):
