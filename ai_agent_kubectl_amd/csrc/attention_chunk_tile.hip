@@ -70,7 +70,9 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
   // operand of weights x values is then one 8-byte LDS read; filled from 16-byte global loads
   bf16_t* VS = reinterpret_cast<bf16_t*>(PG + a.max_blocks);
   __shared__ int s_pos[QT];
-  const int seq = blockIdx.y;
+  // grid (sequences, tiles): the sequence index runs fastest and the tiles run from the last (most keys)
+  // to the first, so the longest workgroups of every sequence start first and the short ones fill in
+  const int seq = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, grp = lane >> 4;
   int row0, nr;
@@ -83,7 +85,7 @@ __global__ __launch_bounds__(NT) void chunk_attention_tile_kernel(bf16_t* __rest
     }
   } else {
     const int q0 = a.q_starts[seq], q1 = a.q_starts[seq + 1];
-    row0 = q0 + QT * blockIdx.x;
+    row0 = q0 + QT * (gridDim.y - 1 - blockIdx.y);
     if (row0 >= q1) return;
     nr = min(QT, q1 - row0);
   }
@@ -353,7 +355,7 @@ int launch(bf16_t* out, const bf16_t* q, const bf16_t* k, const bf16_t* v, const
                                              (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  kern<<<dim3(tiles, a.num_seqs), NT, lds, st>>>(out, q, k, v, a);
+  kern<<<dim3(a.num_seqs, tiles), NT, lds, st>>>(out, q, k, v, a);
   return (int)hipGetLastError();
 }
 
@@ -378,7 +380,7 @@ extern "C" int ka_chunk_attention_tile_ok(int H, int G, int D, int Dv, int BS) {
          Dv == D && (BS & (BS - 1)) == 0 && BS > 0 && lds <= 140 * 1024;
 }
 
-// max_q: the longest run of rows of one sequence in this step (the grid's x extent is ceil(max_q / 16)).
+// max_q: the longest run of rows of one sequence in this step (the grid's y extent is ceil(max_q / 16)).
 // q_starts null: a decode step, token t is the single row of block-table row t (one workgroup per token).
 extern "C" int ka_chunk_attention_tile(void* out, const void* q, const void* k_cache, const void* v_cache,
                                        const int* block_tables, const int* q_starts, int num_seqs, const int* positions,

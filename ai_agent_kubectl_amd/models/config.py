@@ -160,7 +160,9 @@ class VivepelConfig:
         return n
 
     def default_step_tokens(self) -> int:
-        return 4096
+        """16384: the tile attention kernel runs one workgroup per 16 query rows and CU, longest first; a
+        step needs several times 256 of them for the causal tiles' unequal lengths to even out."""
+        return 16384
 
     def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
         return sum(2 * L.mixer.kv_heads * L.mixer.dim * dtype_bytes for L in self.layers)
