@@ -31,10 +31,10 @@
 //     one fragment read per MFMA in the read windows (gb_rp_ab.log).  Rounds 3-4 waited for k-tile
 //     t+1 with a counted vmcnt(16) at a second barrier, keeping t+2's pieces in flight across it:
 //     4-10 % faster, but LDS-DMA pieces do not complete in order and that wait let stale rows through
-//     in some launches (round 5, profiles/r5/gemm_big_clamp/);
+//     in some launches (profiles/r5/gemm_big_clamp/);
 //   * XCD-aware tile order (T1): the bijective round-robin remap, then GM m-tiles x all n-tiles
 //     super-rows so the panels of the tiles running together on one XCD are L2 hits.
-// Measured (round 5, after the drain fix, profiles/r5/gemm_big_clamp/, interleaved with rocBLAS in one
+// Measured (after the drain fix, profiles/r5/gemm_big_clamp/, interleaved with rocBLAS in one
 // process): gate_up + SwiGLU 0.99-1.05x rocBLAS's plain GEMM (+ its separate SiLU pass); QKV on 192-wide
 // tiles 1.01-1.10x at 2048-6144 rows; O / down 0.80-0.92x.  Engine dispatch: EPI_SWIGLU (prefill /
 // mixed-step gate_up, ops.linear_swiglu), EPI_BF16 for QKV where the persisted prefill plan measured it
@@ -212,7 +212,7 @@ KA_DEV void tile_of(int L, int tiles_m, int tiles_n, int gm, int& tm, int& tn) {
 // 16 B, hipMalloc memory); 3: the sc1 loads of 2 after the fences of 1.  hipcc does not pad the
 // VMEM-store-data / VALU-write hazard around asm it cannot see, so the asm stores carry their own
 // wait states (without them a few lanes' data were corrupted: profiles/r4/gemm_big_tail/).
-// Round 5 full-matrix repeats (profiles/r5/gemm_big_tail_modes/): before the LDS-DMA drain fix, modes
+// Full-matrix repeats (profiles/r5/gemm_big_tail_modes/): before the LDS-DMA drain fix, modes
 // 0 and 1 read stale data in some first launches; after it, all four modes were exact in every launch
 // (48 full checks each, after_drain/), so those failures were the DMA hazard.  Mode 2 stays the
 // default because it is the fastest: 2944 x 28672 SwiGLU 639-647 us against 650-667 for the fenced
@@ -597,8 +597,8 @@ __global__ __launch_bounds__(NT, 1) void gemm256_kernel(Args a) {
     // (no lgkmcnt wait here: the next call waits per fragment; the tile's last call waits below)
   };
   // (A five-segment schedule with per-operand counted vmcnt waits, after hipBLASLt's gfx950
-  // MT256x256x64 DirectToLds kernel, measured no faster in round 3 and relied on ordered LDS-DMA
-  // completion: removed in round 5.)
+  // MT256x256x64 DirectToLds kernel, measured no faster and relied on ordered LDS-DMA
+  // completion: removed.)
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
 

@@ -255,7 +255,7 @@ __global__ __launch_bounds__(256) void gemv_ring_kernel(const bf16_t* __restrict
 // KA_GEMV_RING: ring depth 4 (default) or 8, 0 disables the variant (A/B runs).  Measured on
 // MI355X against the staged kernel (profiles/gemv_ring_ab.txt): ring 4 wins O / gate_up at
 // M = 1..4 by 3-10 %, ring 8 is no better, and at M = 16 the staged kernel was faster (QKV 14.5
-// vs 17.9 us) while the X staging loaded one piece per wait.  With the staging batched (round 6,
+// vs 17.9 us) while the X staging loaded one piece per wait.  With the staging batched (
 // profiles/r6/latency_chains/gemv_*): up to 8 rows the 70B TP = 8 rank's B = 8 step is 2.2 % faster on
 // the ring variant and Llama-3-8B's B = 8 within 0.4 %; 16 rows is 1.5 % slower on the 8B.
 #define GEMV_MAX_M 8

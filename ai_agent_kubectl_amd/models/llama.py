@@ -115,7 +115,7 @@ class LlamaModel:
 
     def alloc_cache(self, num_blocks: int, block_size: int):
         """(k_cache [L, NB, Hkv, BS, D], v_cache [L, NB, Hkv, D, BS]) for this rank's KV heads, zero-filled:
-        stale slots read by masked lanes must be finite (attention.hip contract)."""
+        stale slots read by masked lanes must be finite (attention.hip requires it)."""
         L, dt = self.cfg.num_layers, self.W["embed"].dtype
         k = torch.zeros((L, num_blocks, self.hkv, block_size, self.D), dtype=dt, device=self.device)
         v = torch.zeros((L, num_blocks, self.hkv, self.D, block_size), dtype=dt, device=self.device)

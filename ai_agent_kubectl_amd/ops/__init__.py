@@ -512,7 +512,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, split: int = 0, defer_reduce: bool 
 # Prefill / mixed-step gate_up with the SwiGLU epilogue (csrc/gemm_big.hip EPI_SWIGLU): the [M, 2I]
 # gate_up output never exists and the separate SiLU·mul pass goes away.  Every M > TILE_MAX_M (513+)
 # rows (profiles/r3/gemm_big: 565 us vs hipBLASLt 550 us + SiLU·mul at M = 2944, 691 vs 620 + 122
-# at M = 4096, Llama-3-8B; the split tail of round 4 takes the short last round of tiles at smaller
+# at M = 4096, Llama-3-8B; the split tail takes the short last round of tiles at smaller
 # M).  KA_PREFILL_SWIGLU=0 restores hipBLASLt + silu_mul.
 PREFILL_SWIGLU = os.environ.get("KA_PREFILL_SWIGLU", "1") == "1"
 PREFILL_SWIGLU_MIN_M = int(os.environ.get("KA_PREFILL_SWIGLU_MIN_M", "513"))

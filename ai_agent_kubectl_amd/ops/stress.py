@@ -1,6 +1,6 @@
 """Launch-pattern stress checks for the LDS-DMA kernels (race detection on the device).
 
-LDS-DMA pieces of one wave do not always complete in issue order: in round 5 a counted
+LDS-DMA pieces of one wave do not always complete in issue order: a counted
 `s_waitcnt vmcnt(N)` let stale rows through in up to 25 % of `gemm_big` launches, but only under a
 particular launch pattern (each launch right after an unrelated GEMM) and mostly when many lanes of a
 piece read the same address (profiles/r5/gemm_big_clamp/).  This module replays that pattern for the

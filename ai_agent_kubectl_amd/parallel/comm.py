@@ -27,7 +27,7 @@ import torch
 
 # TP decode: the row-parallel O / down projections hand their split-K partials to the fused all-reduce +
 # RMSNorm (csrc/allreduce.hip reduces the slabs while staging its contribution).  0: reduce them first
-# (splitk_reduce), as before round 6.
+# (splitk_reduce).
 TP_SPLITK_NORM = os.environ.get("KA_TP_SPLITK_NORM", "1") == "1"
 
 

@@ -47,7 +47,7 @@ def _worker(rank, world, port, q):
             got_out = ar.all_reduce_rmsnorm(t2, wgt, 1e-5, r2)
             torch.cuda.synchronize()
             errs.append(0.0 if torch.equal(got_out, want_out) and torch.equal(r2, r1) else 1.0)
-            # split-K partial slabs reduced inside the collective (round 6: a TP rank's O / down hand
+            # split-K partial slabs reduced inside the collective (a TP rank's O / down hand
             # their partials to it) == splitk_reduce's bf16 sum then the collective, bit for bit
             for pdt, split in ((torch.float32, 4), (torch.bfloat16, 8), (torch.bfloat16, 2)):
                 slabs = (torch.randn(split, rows, hidden, generator=g) * 0.3).to(pdt).cuda()
