@@ -123,3 +123,21 @@ def test_bench_parallelism_labels():
     assert a.transport == "tcp"
     with pytest.raises(SystemExit):
         bench.parse_args(["--gpus", "4", "--tp", "3"])
+
+
+def test_arch_compare_is_an_option_and_off_by_default():
+    """`--arch-compare` (Vivepel beside Llama at equal sizes) leaves the default workload alone."""
+    import importlib.util
+    import os
+
+    spec = importlib.util.spec_from_file_location("bench_main", os.path.join(os.path.dirname(__file__), "..", "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    a = bench.parse_args([])
+    assert a.arch_compare is False and a.model == os.environ.get("BENCH_MODEL", "llama3-8b") and a.gpus == 1
+    b = bench.parse_args(["--arch-compare", "--arch-sizes", "2k"])
+    assert b.arch_compare is True and b.arch_sizes == "2k"
+    from ai_agent_kubectl_amd import bench_arch
+    ll, vv = bench_arch._configs("2k", 512)
+    assert (ll.hidden, ll.num_heads, ll.intermediate) == (vv.hidden, vv.layers[0].mixer.heads, vv.layers[0].ff)
+    assert vv.layers[0].mixer.chunk == 512 and vv.num_layers == ll.num_layers

@@ -518,24 +518,37 @@ def test_bf16_engine_tile_kernel_shapes(tmp_path):
 
 
 @pytest.mark.gpu
-def test_graph_decode_matches_eager(tmp_path):
-    """Captured decode graphs (replayed several times, with eager steps between) give the eager tokens."""
+@pytest.mark.parametrize("kind", ["fp32_small_heads", "bf16_tile_kernel"])
+def test_graph_decode_matches_eager(tmp_path, kind):
+    """Captured decode graphs (replayed many times, with eager prompt steps between) give the eager
+    tokens: the per-token attention kernel in fp32, and the tile kernel's one-row form in bf16 (head size
+    32, more dynamic LDS than the default limit)."""
     from ai_agent_kubectl_amd.engine.builder import EngineOptions, build_engine
     from ai_agent_kubectl_amd.engine.sequence import SamplingParams
 
-    config = variant("base")
+    if kind == "fp32_small_heads":
+        config, dtype = variant("base"), "float32"
+    else:
+        g = torch.Generator().manual_seed(3)
+        config = oracle.random_config(g, layers=2, width=64, vocab=272, groups=2, heads=20, kv_heads=4, dim=32, vdim=32,
+                                      rot={"base": 1000.0, "dims": 16}, mask={"size": 24}, scale=0.2, softcap=15.0)
+        dtype = "bfloat16"
     W = oracle.random_weights(config, seed=19)
     path = write_checkpoint(tmp_path / "m", config, W)
     prompts = [tokens_for(config, n, seed=40 + n) for n in (6, 17, 11)]
     outs = []
     for graphs in (False, True):
-        eng = build_engine(EngineOptions(model=path, device="cuda", dtype="float32", max_batch=4, max_model_len=96,
+        eng = build_engine(EngineOptions(model=path, device="cuda", dtype=dtype, max_batch=4, max_model_len=96,
                                          kv_cache_tokens=256, graph_buckets=(1, 2, 4), safe_decode=False,
                                          ignore_eos=True, use_graphs=graphs))
         if graphs:
             eng.runner.capture_graphs()
-        seqs = eng.generate_blocking(prompts, SamplingParams(max_new_tokens=24, ignore_eos=True, safe_decode=False))
+        got = []
+        for _ in range(2):      # a second wave reuses the freed pages and replays the same graphs
+            seqs = eng.generate_blocking(prompts, SamplingParams(max_new_tokens=24, ignore_eos=True, safe_decode=False))
+            got.append([s.generated for s in seqs])
         if graphs:
             assert eng.runner.stats["graph_replays"] > 0
-        outs.append([s.generated for s in seqs])
+        assert got[0] == got[1]
+        outs.append(got[0])
     assert outs[0] == outs[1]
