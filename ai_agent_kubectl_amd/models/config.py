@@ -74,7 +74,7 @@ class AttentionSpec:
     kv_heads: int
     dim: int                    # per-head query / key size
     vdim: int                   # per-head value size (the values are the projected keys: vdim == dim)
-    chunk: int                  # chunked causal mask: position p sees floor(p / chunk) * chunk .. p
+    chunk: int                  # chunked causal mask: position p sees floor(p / chunk) * chunk .. p (0: all of 0 .. p)
     rot_dims: int               # rotary positions on the first rot_dims entries of each head
     rot_base: float
     scale: float
@@ -82,14 +82,17 @@ class AttentionSpec:
 
     @classmethod
     def from_dict(cls, m: dict) -> "AttentionSpec":
+        mask, rot, cap = m.get("mask"), m.get("rot"), m.get("softcap")
         spec = cls(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
-                   chunk=int(m["mask"]["size"]), rot_dims=int(m["rot"]["dims"]), rot_base=float(m["rot"]["base"]),
-                   scale=float(m["scale"]), softcap=float(m["softcap"]))
+                   chunk=int(mask["size"]) if mask else 0,            # no mask entry: plain causal
+                   rot_dims=int(rot["dims"]) if rot else 0,           # no rot entry: no rotary positions
+                   rot_base=float(rot["base"]) if rot else 1.0,
+                   scale=float(m["scale"]), softcap=float(cap) if cap else 0.0)   # no softcap: scores as they are
         if spec.heads % spec.kv_heads:
             raise ValueError(f"heads {spec.heads} must be a multiple of kv_heads {spec.kv_heads}")
         if spec.vdim != spec.dim:
             raise ValueError(f"vdim {spec.vdim} != dim {spec.dim}: the values are the projected keys")
-        if spec.rot_dims % 2 or spec.rot_dims > spec.dim or spec.chunk <= 0:
+        if spec.rot_dims % 2 or spec.rot_dims > spec.dim or spec.chunk < 0:
             raise ValueError(f"bad rotary dims {spec.rot_dims} / chunk {spec.chunk} for head size {spec.dim}")
         return spec
 
@@ -144,7 +147,7 @@ class VivepelConfig:
                 "norm": {"eps": self.norm_eps, "groups": self.norm_groups},
                 "layers": [{"type": "attention",
                             "mixer": {"heads": L.mixer.heads, "kv_heads": L.mixer.kv_heads, "dim": L.mixer.dim,
-                                      "vdim": L.mixer.vdim, "mask": {"size": L.mixer.chunk},
+                                      "vdim": L.mixer.vdim, "mask": {"size": L.mixer.chunk} if L.mixer.chunk else None,
                                       "rot": {"base": L.mixer.rot_base, "dims": L.mixer.rot_dims},
                                       "scale": L.mixer.scale, "softcap": L.mixer.softcap},
                             "mlp": {"kind": "dense", "ff": L.ff} if L.ff else None} for L in self.layers]}

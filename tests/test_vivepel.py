@@ -469,6 +469,23 @@ def test_steps_that_want_nothing(tmp_path, device):
     assert sess.engine.bm.num_free == sess.engine.bm.num_blocks
 
 
+@pytest.mark.parametrize("device", DEVICES)
+def test_layer_without_mask_rot_or_softcap_entries(tmp_path, device):
+    """A mixer whose configuration leaves out the mask, the rotary entry and the soft cap: plain causal
+    attention (still with the sink and the head mixing).  The oracle gets the equivalent explicit values."""
+    config = variant("base")
+    W = oracle.random_weights(config, seed=23)
+    lean = json.loads(json.dumps(config))
+    for L in lean["layers"][:1]:
+        del L["mixer"]["mask"], L["mixer"]["rot"], L["mixer"]["softcap"]
+    full = json.loads(json.dumps(config))
+    full["layers"][0]["mixer"].update(mask={"size": 1 << 20}, rot={"base": 1.0, "dims": 0}, softcap=1e9)
+    sess = session(write_checkpoint(tmp_path / "m", lean, W), device)
+    toks = tokens_for(config, 40, seed=11)
+    got = replay(sess, toks, [13, 2, 20] + [1] * 5)
+    assert rel_err(got, want_logits(full, W, toks)) < tol("float32")
+
+
 def test_settings_select_a_checkpoint_folder_and_dtype(tmp_path):
     from ai_agent_kubectl_amd.config import Settings
     from ai_agent_kubectl_amd.engine.builder import EngineOptions
