@@ -96,7 +96,8 @@ class VivepelModel:
                                             m.rot_dims, eps)
             a = mixers.chunk_attention(q, k_cache[li], v_cache[li], meta.block_tables, q_starts, meta.positions,
                                        meta.slot_mapping, L["talk"], m.chunk, m.scale, m.softcap, sink=True,
-                                       max_q=0 if meta.is_decode else meta.max_q_len)
+                                       max_q=0 if meta.is_decode else meta.max_q_len,
+                                       num_decode=0 if meta.is_decode else meta.num_decode)
             y = F.linear(a, L["wo"])
             nxt = self.layers[li + 1]["norm1"] if li < last else None
             if spec.ff:

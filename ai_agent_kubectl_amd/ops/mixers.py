@@ -119,7 +119,7 @@ def headnorm_rope_append(qk: torch.Tensor, q_w: torch.Tensor, k_w: torch.Tensor,
 def chunk_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     q_starts: Optional[torch.Tensor], positions: torch.Tensor, slots: torch.Tensor,
                     mix: Optional[torch.Tensor], chunk: int, scale: float, cap: float, sink: bool,
-                    max_q: int = 0) -> torch.Tensor:
+                    max_q: int = 0, num_decode: int = 0) -> torch.Tensor:
     """q [T, H, D] -> [T, H * Dv].  q_starts [S + 1]: first row of each sequence in a varlen step (rows
     past q_starts[S] must be padding, slot < 0); None: token t is block-table row t (a decode step).  chunk 0: plain causal; cap 0: no soft cap; mix None: no head mixing."""
     if _ref(q):
@@ -140,10 +140,19 @@ def chunk_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         # decode (q_starts None): one workgroup per token writes every row
         varlen = q_starts is not None
         out = (torch.zeros if varlen else torch.empty)((T, H * Dv), dtype=q.dtype, device=q.device)
-        check(lib.ka_chunk_attention_tile(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(q_starts),
-                                          block_tables.shape[0] if varlen else T, _p(positions), _p(slots), _p(mix),
-                                          int(max_q) if varlen else 1, H, G, D, Dv, int(chunk), BS, block_tables.shape[1],
-                                          int(bool(sink)), float(scale), float(cap), _stream()), "chunk_attention_tile")
+        tail = (H, G, D, Dv, int(chunk), BS, block_tables.shape[1], int(bool(sink)), float(scale), float(cap), _stream())
+        nd = min(int(num_decode), block_tables.shape[0]) if varlen else 0
+        if nd > 0:   # the leading one-token sequences: token t is block-table row t
+            check(lib.ka_chunk_attention_tile(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), None, nd,
+                                              _p(positions), _p(slots), _p(mix), 1, *tail), "chunk_attention_tile")
+        S = block_tables.shape[0] - nd
+        if not varlen:
+            check(lib.ka_chunk_attention_tile(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), None, T,
+                                              _p(positions), _p(slots), _p(mix), 1, *tail), "chunk_attention_tile")
+        elif S > 0:   # (q_starts holds absolute rows, so the remaining sequences index q and out as they are)
+            check(lib.ka_chunk_attention_tile(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables[nd:]),
+                                              _p(q_starts[nd:]), S, _p(positions), _p(slots), _p(mix), int(max_q), *tail),
+                  "chunk_attention_tile")
         return out
     out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
     check(lib.ka_chunk_attention(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(q_starts),

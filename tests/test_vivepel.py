@@ -532,6 +532,13 @@ def test_bf16_engine_tile_kernel_shapes(tmp_path):
     want = want_logits(config, W, toks)
     assert rel_err(replay(sess, toks, [len(toks)]), want) < tol("bfloat16")
     assert rel_err(replay(sess, toks, [9, 17, 30, 2, 16, 1]), want) < tol("bfloat16")
+    # a mixed step: decode rows of two requests (the one-row form) beside a 40-row portion of a third (16-row tiles)
+    other = tokens_for(config, 40, seed=12)
+    sess.step([{"id": "a", "tokens": toks[:20], "want": []}, {"id": "b", "tokens": toks[:33], "want": []}], [])
+    got = sess.step([{"id": "a", "tokens": toks[20:21], "want": [0]}, {"id": "c", "tokens": other, "want": list(range(40))},
+                     {"id": "b", "tokens": toks[33:34], "want": [0]}], ["a", "b", "c"])
+    assert rel_err(got[0:1], want[20:21]) < tol("bfloat16") and rel_err(got[41:42], want[33:34]) < tol("bfloat16")
+    assert rel_err(got[1:41], want_logits(config, W, other)) < tol("bfloat16")
 
 
 @pytest.mark.gpu
