@@ -1,0 +1,283 @@
+// KA_HIP_LIB: mixers
+// KA_HIPCC_FLAGS: -Xclang -target-feature -Xclang -packed-fp32-ops
+// Latent attention over a paged cache (models/kafilorn.py).  A token's cache entry is one row
+// [R + Dr]: the RMS-normed key/value latent c [R] and one rotated key part k_r [Dr] shared by all heads;
+// the per-head keys W_uk c and values W_uv c are never materialised: the query is carried into the latent
+// space (q_lat = W_uk^T q, a batched GEMM outside), the attention runs multi-query over the rows with the
+// latent itself as the value, and W_uv is applied to the result (another batched GEMM outside).
+//
+//   latent_prep:   from the fused down-projection row [Q | R | Dr]: the RMS-normed query latent [Q]; the
+//                  RMS-normed c and the rotated k_r appended to the cache at the token's slot.
+//   rope_split_q:  q [T, H, D + Dr] -> the unrotated parts [H, T, D] (the batched GEMM's operand layout) and
+//                  the rotated parts [T, H, Dr] in fp32.  Rotary: entry i pairs with i + dims/2 among the
+//                  first `dims` entries, angle = position * inv_freq[i].
+//   window_attention:  s_h(j) = (q_lat_h . c_j + q_rot_h . k_r,j) * scale for the keys j with
+//                  0 <= p - j < window (window 0: all j <= p); weights exp(s) / (sum exp(s) + exp(sink_h)),
+//                  the sink optional; out_h = sum_j w_h(j) c_j, written [H, T, R].
+//                  One workgroup per (token, group of heads); keys in tiles of 64 with an online softmax in
+//                  fp32.  A decode step is the same launch with one token per sequence.
+#include "rows_f32.h"
+
+namespace {
+using namespace rows;
+
+constexpr int KT = 64;
+constexpr int MAX_ACC = 32;   // outputs per thread: heads per workgroup * R <= NT * MAX_ACC
+
+KA_DEV float rot_entry(float self, float partner, bool first_half, float ang) {
+  float sn, cs;
+  sincosf(ang, &sn, &cs);
+  return first_half ? self * cs - partner * sn : self * cs + partner * sn;
+}
+
+template <typename AT>
+__global__ __launch_bounds__(NT) void latent_prep_kernel(AT* __restrict__ cq, const AT* __restrict__ proj, int P, int Q,
+                                                         int R, int Dr, const float* __restrict__ w_q,
+                                                         const float* __restrict__ w_kv, const float* __restrict__ inv_freq,
+                                                         const int* __restrict__ positions, const int* __restrict__ slots,
+                                                         AT* __restrict__ cache, int rot_dims, float eps) {
+  __shared__ float red[NW];
+  const int t = blockIdx.x;
+  const AT* row = proj + (size_t)t * P;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < Q; i += NT) {
+    const float v = ldf(row + i);
+    s += v * v;
+  }
+  float inv = 1.0f / sqrtf(block_sum(s, red) / (float)Q + eps);
+  for (int i = threadIdx.x; i < Q; i += NT) stf(cq + (size_t)t * Q + i, ldf(row + i) * inv * w_q[i]);
+  if (cache == nullptr) return;
+  const int slot = slots[t];
+  if (slot < 0) return;
+  s = 0.f;
+  for (int i = threadIdx.x; i < R; i += NT) {
+    const float v = ldf(row + Q + i);
+    s += v * v;
+  }
+  inv = 1.0f / sqrtf(block_sum(s, red) / (float)R + eps);
+  AT* dst = cache + (size_t)slot * (R + Dr);
+  for (int i = threadIdx.x; i < R; i += NT) stf(dst + i, ldf(row + Q + i) * inv * w_kv[i]);
+  const int half = rot_dims >> 1;
+  const float pos = (float)positions[t];
+  const AT* kr = row + Q + R;
+  for (int i = threadIdx.x; i < Dr; i += NT) {
+    float o = ldf(kr + i);
+    if (i < rot_dims) {
+      const int j = i < half ? i : i - half;
+      o = rot_entry(o, ldf(kr + (i < half ? i + half : i - half)), i < half, pos * inv_freq[j]);
+    }
+    stf(dst + R + i, o);
+  }
+}
+
+template <typename AT>
+__global__ __launch_bounds__(NT) void rope_split_q_kernel(AT* __restrict__ qn, float* __restrict__ qr,
+                                                          const AT* __restrict__ q, const float* __restrict__ inv_freq,
+                                                          const int* __restrict__ positions, int T, int H, int D, int Dr,
+                                                          int rot_dims) {
+  const int t = blockIdx.x;
+  const int half = rot_dims >> 1, DD = D + Dr;
+  const float pos = (float)positions[t];
+  const AT* row = q + (size_t)t * H * DD;
+  for (int idx = threadIdx.x; idx < H * DD; idx += NT) {
+    const int h = idx / DD, i = idx % DD;
+    if (i < D) {
+      qn[((size_t)h * T + t) * D + i] = row[idx];
+    } else {
+      const int e = i - D;
+      float o = ldf(row + idx);
+      if (e < rot_dims) {
+        const int j = e < half ? e : e - half;
+        o = rot_entry(o, ldf(row + h * DD + D + (e < half ? e + half : e - half)), e < half, pos * inv_freq[j]);
+      }
+      qr[((size_t)t * H + h) * Dr + e] = o;
+    }
+  }
+}
+
+struct WinArgs {
+  const int* block_tables;   // [S, max_blocks]
+  const int* q_starts;       // [S + 1] or null
+  int num_seqs;
+  const int* positions;      // [T]
+  const int* slots;          // [T] < 0: padding row
+  const float* sink;         // [H] or null
+  int T, H, HG, R, Dr, BS, max_blocks, window;
+  float scale;
+};
+
+template <typename AT>
+__global__ __launch_bounds__(NT) void window_attention_kernel(AT* __restrict__ out, const AT* __restrict__ q_lat,
+                                                              const float* __restrict__ q_rot,
+                                                              const AT* __restrict__ cache, WinArgs a) {
+  extern __shared__ float lds[];
+  const int R = a.R, Dr = a.Dr, E = R + Dr, HG = a.HG, H = a.H, T = a.T;
+  float* ql = lds;                 // [HG][E]  query in the latent space, then its rotated part
+  float* sc = ql + HG * E;         // [HG][KT] scores, then unnormalised weights of the tile
+  float* corr = sc + HG * KT;      // [HG] rescale of the accumulators for the tile
+  float* linv = corr + HG;         // [HG] 1 / denominator at the end
+  __shared__ int page[KT];
+  const int t = blockIdx.x, h0 = blockIdx.y * HG;
+  const int hg = min(HG, H - h0);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (a.slots[t] < 0) {
+    for (int i = threadIdx.x; i < hg * R; i += NT) stf(out + ((size_t)(h0 + i / R) * T + t) * R + i % R, 0.f);
+    return;
+  }
+  const int p = a.positions[t];
+  const int seq = seq_of(a.q_starts, a.num_seqs, t);
+  const int* bt = a.block_tables + (size_t)seq * a.max_blocks;
+  const int start = a.window > 0 ? max(0, p - a.window + 1) : 0;
+  const int n = p - start + 1;
+  for (int i = threadIdx.x; i < hg * E; i += NT) {
+    const int g = i / E, e = i % E;
+    ql[i] = e < R ? ldf(q_lat + ((size_t)(h0 + g) * T + t) * R + e) : q_rot[((size_t)t * H + h0 + g) * Dr + e - R];
+  }
+  // running maximum and denominator per head live in the registers of the head's wave (head g: wave g % NW)
+  float run_m[16], run_l[16];
+#pragma unroll
+  for (int u = 0; u < 16; ++u) {
+    const int g = wave + u * NW;
+    const bool sk = a.sink != nullptr && g < hg;
+    run_m[u] = sk ? a.sink[h0 + g] : -INFINITY;
+    run_l[u] = sk ? 1.f : 0.f;
+  }
+  float acc[MAX_ACC];
+#pragma unroll
+  for (int u = 0; u < MAX_ACC; ++u) acc[u] = 0.f;
+  const int BS = a.BS;
+  for (int k0 = 0; k0 < n; k0 += KT) {
+    const int nk = min(KT, n - k0);
+    __syncthreads();
+    if (threadIdx.x < nk) page[threadIdx.x] = bt[(start + k0 + threadIdx.x) / BS];
+    __syncthreads();
+    for (int it = threadIdx.x; it < hg * KT; it += NT) {
+      const int g = it / KT, j = it % KT;
+      float s = -INFINITY;
+      if (j < nk) {
+        const int pos = start + k0 + j;
+        const AT* kr = cache + ((size_t)page[j] * BS + pos % BS) * E;
+        const float* qg = ql + g * E;
+        s = 0.f;
+        if constexpr (sizeof(AT) == 2) {
+          if ((E & 7) == 0) {
+            for (int i = 0; i < E; i += 8) {
+              const uint4 kv = *reinterpret_cast<const uint4*>(kr + i);
+              const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + i), qb = *reinterpret_cast<const f32x4*>(qg + i + 4);
+              s += qa[0] * lo_f(kv.x) + qa[1] * hi_f(kv.x) + qa[2] * lo_f(kv.y) + qa[3] * hi_f(kv.y) +
+                   qb[0] * lo_f(kv.z) + qb[1] * hi_f(kv.z) + qb[2] * lo_f(kv.w) + qb[3] * hi_f(kv.w);
+            }
+          } else {
+            for (int i = 0; i < E; ++i) s += qg[i] * ldf(kr + i);
+          }
+        } else {
+          if ((E & 3) == 0) {
+            for (int i = 0; i < E; i += 4) {
+              const f32x4 kv = *reinterpret_cast<const f32x4*>(kr + i);
+              const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + i);
+              s += qa[0] * kv[0] + qa[1] * kv[1] + qa[2] * kv[2] + qa[3] * kv[3];
+            }
+          } else {
+            for (int i = 0; i < E; ++i) s += qg[i] * ldf(kr + i);
+          }
+        }
+        s *= a.scale;
+      }
+      sc[it] = s;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int g = wave + u * NW;
+      if (g < hg) {
+        const float s = sc[g * KT + lane];
+        const float m = fmaxf(run_m[u], wave_max(s));
+        const float e = s == -INFINITY ? 0.f : expf(s - m);
+        const float c = run_m[u] == -INFINITY ? 0.f : expf(run_m[u] - m);
+        run_l[u] = run_l[u] * c + wave_sum(e);
+        run_m[u] = m;
+        sc[g * KT + lane] = e;
+        if (lane == 0) corr[g] = c;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < MAX_ACC; ++u) {
+      const int i = threadIdx.x + u * NT;
+      if (i < hg * R) {
+        const int g = i / R, r = i % R;
+        const float* wg = sc + g * KT;
+        float s = acc[u] * corr[g];
+        for (int j = 0; j < nk; ++j) {
+          const int pos = start + k0 + j;
+          s += wg[j] * ldf(cache + ((size_t)page[j] * BS + pos % BS) * E + r);
+        }
+        acc[u] = s;
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < 16; ++u) {
+    const int g = wave + u * NW;
+    if (g < hg && lane == 0) linv[g] = 1.0f / run_l[u];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < MAX_ACC; ++u) {
+    const int i = threadIdx.x + u * NT;
+    if (i < hg * R) stf(out + ((size_t)(h0 + i / R) * T + t) * R + i % R, acc[u] * linv[i / R]);
+  }
+}
+
+}  // namespace
+
+extern "C" int ka_latent_prep(void* cq, const void* proj, int T, int P, int Q, int R, int Dr, const float* w_q,
+                              const float* w_kv, const float* inv_freq, const int* positions, const int* slots,
+                              void* cache, int rot_dims, float eps, int f32, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (Q <= 0 || P < Q || (cache != nullptr && (P < Q + R + Dr || R <= 0)) || rot_dims < 0 || rot_dims > Dr || (rot_dims & 1))
+    return (int)hipErrorInvalidValue;
+  if (f32)
+    latent_prep_kernel<float><<<T, NT, 0, st>>>((float*)cq, (const float*)proj, P, Q, R, Dr, w_q, w_kv, inv_freq, positions,
+                                                slots, (float*)cache, rot_dims, eps);
+  else
+    latent_prep_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)cq, (const bf16_t*)proj, P, Q, R, Dr, w_q, w_kv, inv_freq,
+                                                 positions, slots, (bf16_t*)cache, rot_dims, eps);
+  KA_CHECK_LAUNCH();
+}
+
+extern "C" int ka_rope_split_q(void* qn, float* qr, const void* q, const float* inv_freq, const int* positions, int T,
+                               int H, int D, int Dr, int rot_dims, int f32, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (rot_dims < 0 || rot_dims > Dr || (rot_dims & 1)) return (int)hipErrorInvalidValue;
+  if (f32) rope_split_q_kernel<float><<<T, NT, 0, st>>>((float*)qn, qr, (const float*)q, inv_freq, positions, T, H, D, Dr, rot_dims);
+  else rope_split_q_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)qn, qr, (const bf16_t*)q, inv_freq, positions, T, H, D, Dr, rot_dims);
+  KA_CHECK_LAUNCH();
+}
+
+extern "C" int ka_window_attention(void* out, const void* q_lat, const float* q_rot, const void* cache,
+                                   const int* block_tables, const int* q_starts, int num_seqs, const int* positions,
+                                   const int* slots, const float* sink, int T, int H, int R, int Dr, int BS,
+                                   int max_blocks, int window, float scale, int f32, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (H <= 0 || R <= 0 || Dr < 0 || BS <= 0 || window < 0 || R > NT * MAX_ACC) return (int)hipErrorInvalidValue;
+  // heads per workgroup: as many as the accumulators (NT * MAX_ACC outputs), the 16 running values per wave
+  // and 120 KB of LDS allow
+  int HG = min(H, min(NT * MAX_ACC / R, 16 * NW));
+  while (HG > 1 && (size_t)(HG * (R + Dr + KT + 2)) * sizeof(float) > 120 * 1024) --HG;
+  const size_t lds = (size_t)(HG * (R + Dr + KT + 2)) * sizeof(float);
+  if (lds > 120 * 1024) return (int)hipErrorInvalidValue;
+  WinArgs a{block_tables, q_starts, num_seqs, positions, slots, sink, T, H, HG, R, Dr, BS, max_blocks, window, scale};
+  const void* fn = f32 ? reinterpret_cast<const void*>(window_attention_kernel<float>)
+                       : reinterpret_cast<const void*>(window_attention_kernel<bf16_t>);
+  if (lds > 48 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+  }
+  dim3 grid(T, (H + HG - 1) / HG);
+  if (f32)
+    window_attention_kernel<float><<<grid, NT, lds, st>>>((float*)out, (const float*)q_lat, q_rot, (const float*)cache, a);
+  else
+    window_attention_kernel<bf16_t><<<grid, NT, lds, st>>>((bf16_t*)out, (const bf16_t*)q_lat, q_rot, (const bf16_t*)cache, a);
+  KA_CHECK_LAUNCH();
+}

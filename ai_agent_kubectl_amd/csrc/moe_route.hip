@@ -1,0 +1,185 @@
+// KA_HIP_LIB: mixers
+// KA_HIPCC_FLAGS: -Xclang -target-feature -Xclang -packed-fp32-ops
+// Mixture-of-experts routing with expert groups and a choice correction, and the experts of a few rows
+// (models/kafilorn.py).
+//
+//   moe_route:  z = W_router h in fp32 (weights [E, W] fp32, one wave per logit); s = softmax(z) over all
+//               experts; choice = s + correction (optional).  The experts form `groups` equal groups of
+//               neighbours; a group's score is its largest choice; only experts of the `keep` best groups
+//               can be chosen.  The `top` largest choices are taken (ties: the lower index); the weights
+//               are their s (without the correction) over their sum (+ 1e-20).  One workgroup per token.
+//   moe_gate_up / moe_down:  for step sizes of a few rows (decode), the chosen experts as matrix-vector
+//               products straight from the stacked expert weights, no routing lists and no host read, so a
+//               decode step can be captured: act[t, k] = silu(gate_e h) * (up_e h) with e = ids[t, k], then
+//               out[t] = sum_k w[t, k] down_e act[t, k] in fp32.
+#include "rows_f32.h"
+
+namespace {
+using namespace rows;
+
+constexpr int MAX_E = 1024;
+constexpr int MAX_TOP = 32;
+
+template <typename AT>
+__global__ __launch_bounds__(NT) void moe_route_kernel(int* __restrict__ ids, float* __restrict__ wts,
+                                                       const AT* __restrict__ h, const float* __restrict__ wr,
+                                                       const float* __restrict__ correction, int width, int E, int top,
+                                                       int groups, int keep) {
+  __shared__ float z[MAX_E];      // logits, then scores
+  __shared__ float ch[MAX_E];     // choice scores (minus infinity once taken or outside the kept groups)
+  __shared__ float gs[MAX_E];     // group scores
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const AT* hr = h + (size_t)t * width;
+  for (int e = wave; e < E; e += NW) {
+    const float* we = wr + (size_t)e * width;
+    float s = 0.f;
+    for (int i = lane; i < width; i += 64) s += ldf(hr + i) * we[i];
+    s = wave_sum(s);
+    if (lane == 0) z[e] = s;
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  float mx = -INFINITY;
+  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += 64) sum += expf(z[e] - mx);
+  sum = wave_sum(sum);
+  for (int e = lane; e < E; e += 64) {
+    const float s = expf(z[e] - mx) / sum;
+    z[e] = s;
+    ch[e] = s + (correction != nullptr ? correction[e] : 0.f);
+  }
+  __builtin_amdgcn_wave_barrier();
+  const int per = E / groups;
+  if (groups > 1) {
+    for (int g = lane; g < groups; g += 64) {
+      float b = -INFINITY;
+      for (int e = g * per; e < (g + 1) * per; ++e) b = fmaxf(b, ch[e]);
+      gs[g] = b;
+    }
+    __builtin_amdgcn_wave_barrier();
+    // a group is kept when fewer than `keep` groups come before it (larger score, or equal and lower index)
+    for (int g = lane; g < groups; g += 64) {
+      int before = 0;
+      for (int o = 0; o < groups; ++o) before += (gs[o] > gs[g] || (gs[o] == gs[g] && o < g)) ? 1 : 0;
+      if (before >= keep)
+        for (int e = g * per; e < (g + 1) * per; ++e) ch[e] = -INFINITY;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  float wsum = 0.f, mine = 0.f;
+  int mid = 0;
+  for (int k = 0; k < top; ++k) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64)
+      if (ch[e] > bv) { bv = ch[e]; bi = e; }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(bv, off, 64);
+      const int oi = __shfl_xor(bi, off, 64);
+      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if (bi >= E) bi = 0;   // fewer finite choices than `top`: cannot happen for a valid router
+    const float s = z[bi];
+    wsum += s;
+    if (lane == k % 64) { mine = s; mid = bi; }   // top <= MAX_TOP <= 64: lane k keeps the k-th choice
+    if (lane == 0) ch[bi] = -INFINITY;
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (lane < top) {
+    ids[(size_t)t * top + lane] = mid;
+    wts[(size_t)t * top + lane] = mine / (wsum + 1e-20f);
+  }
+}
+
+// act[row, f] for row = t * top + k: one workgroup per (row, 4 * FPW outputs), h staged in LDS as fp32
+constexpr int FPW = 4;   // outputs per wave
+template <typename AT>
+__global__ __launch_bounds__(NT) void moe_gate_up_kernel(AT* __restrict__ act, const AT* __restrict__ h,
+                                                         const AT* __restrict__ w_gu, const int* __restrict__ ids,
+                                                         int width, int ff, int top) {
+  extern __shared__ float hs[];   // [width]
+  const int row = blockIdx.x, t = row / top;
+  const int e = ids[row];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < width; i += NT) hs[i] = ldf(h + (size_t)t * width + i);
+  __syncthreads();
+  const AT* wg = w_gu + (size_t)e * 2 * ff * width;
+  for (int u = 0; u < FPW; ++u) {
+    const int f = (blockIdx.y * NW + wave) * FPW + u;
+    if (f >= ff) break;
+    const AT* g = wg + (size_t)f * width;
+    const AT* up = wg + (size_t)(ff + f) * width;
+    float sg = 0.f, su = 0.f;
+    for (int i = lane; i < width; i += 64) {
+      sg += hs[i] * ldf(g + i);
+      su += hs[i] * ldf(up + i);
+    }
+    sg = wave_sum(sg);
+    su = wave_sum(su);
+    if (lane == 0) stf(act + (size_t)row * ff + f, sg / (1.f + expf(-sg)) * su);
+  }
+}
+
+// out[t, c] = sum_k w[t, k] * (down_e[c, :] . act[t * top + k, :]): one workgroup per (t, 4 * FPW columns)
+template <typename AT>
+__global__ __launch_bounds__(NT) void moe_down_kernel(float* __restrict__ out, const AT* __restrict__ act,
+                                                      const AT* __restrict__ w_down, const int* __restrict__ ids,
+                                                      const float* __restrict__ wts, int width, int ff, int top) {
+  extern __shared__ float as[];   // [top][ff]
+  __shared__ int se[MAX_TOP];
+  __shared__ float sw[MAX_TOP];
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < top * ff; i += NT) as[i] = ldf(act + (size_t)t * top * ff + i);
+  if (threadIdx.x < top) {
+    se[threadIdx.x] = ids[(size_t)t * top + threadIdx.x];
+    sw[threadIdx.x] = wts[(size_t)t * top + threadIdx.x];
+  }
+  __syncthreads();
+  for (int u = 0; u < FPW; ++u) {
+    const int c = (blockIdx.y * NW + wave) * FPW + u;
+    if (c >= width) break;
+    float s = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const AT* d = w_down + ((size_t)se[k] * width + c) * ff;
+      float p = 0.f;
+      for (int i = lane; i < ff; i += 64) p += as[k * ff + i] * ldf(d + i);
+      s += sw[k] * p;
+    }
+    s = wave_sum(s);
+    if (lane == 0) out[(size_t)t * width + c] = s;
+  }
+}
+
+}  // namespace
+
+extern "C" int ka_moe_route(int* ids, float* wts, const void* h, const float* wr, const float* correction, int T,
+                            int width, int E, int top, int groups, int keep, int f32, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (E <= 0 || E > MAX_E || top <= 0 || top > MAX_TOP || top > E || groups <= 0 || E % groups || keep <= 0 || keep > groups)
+    return (int)hipErrorInvalidValue;
+  if (f32) moe_route_kernel<float><<<T, NT, 0, st>>>(ids, wts, (const float*)h, wr, correction, width, E, top, groups, keep);
+  else moe_route_kernel<bf16_t><<<T, NT, 0, st>>>(ids, wts, (const bf16_t*)h, wr, correction, width, E, top, groups, keep);
+  KA_CHECK_LAUNCH();
+}
+
+extern "C" int ka_moe_rows(float* out, void* act, const void* h, const void* w_gu, const void* w_down, const int* ids,
+                           const float* wts, int T, int width, int ff, int top, int f32, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (top <= 0 || top > MAX_TOP || (size_t)width * 4 > 60 * 1024 || (size_t)top * ff * 4 > 60 * 1024)
+    return (int)hipErrorInvalidValue;
+  const int per = NW * FPW;
+  dim3 g1(T * top, (ff + per - 1) / per), g2(T, (width + per - 1) / per);
+  const size_t l1 = (size_t)width * sizeof(float), l2 = (size_t)top * ff * sizeof(float);
+  if (f32) {
+    moe_gate_up_kernel<float><<<g1, NT, l1, st>>>((float*)act, (const float*)h, (const float*)w_gu, ids, width, ff, top);
+    moe_down_kernel<float><<<g2, NT, l2, st>>>(out, (const float*)act, (const float*)w_down, ids, wts, width, ff, top);
+  } else {
+    moe_gate_up_kernel<bf16_t><<<g1, NT, l1, st>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, ids, width, ff, top);
+    moe_down_kernel<bf16_t><<<g2, NT, l2, st>>>(out, (const bf16_t*)act, (const bf16_t*)w_down, ids, wts, width, ff, top);
+  }
+  KA_CHECK_LAUNCH();
+}

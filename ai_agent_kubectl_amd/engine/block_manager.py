@@ -227,6 +227,31 @@ class BlockManager:
         self.cached = {h: b for h, b in self.cached.items() if self.ref[b] > 0}
 
 
+class StateSlots:
+    """Slots of per-sequence recurrent state (models whose mixers carry a state from token to token, beside or
+    instead of paged keys): a fixed pool, one slot per live sequence, taken at admission and given back when the
+    sequence finishes, is aborted or is preempted.  A slot's contents are not cleared: the model starts a
+    sequence's first row (position 0) from the zero state."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self.free = collections.deque(range(num_slots))
+
+    @property
+    def num_free(self) -> int:
+        return len(self.free)
+
+    def acquire(self) -> int:
+        if not self.free:
+            raise NoFreeBlocks("no free state slot")
+        return self.free.popleft()
+
+    def release(self, slot: int) -> None:
+        if slot >= 0:
+            assert slot not in self.free
+            self.free.append(slot)
+
+
 def make_block_manager(num_blocks: int, block_size: int = 16, enable_prefix_caching: bool = True):
     """The C++ allocator (runtime/native.cpp) when built, else this Python reference."""
     try:

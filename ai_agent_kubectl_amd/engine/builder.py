@@ -46,6 +46,7 @@ class EngineOptions:
     ignore_eos: bool = False
     prefix_caching: bool = True
     dtype: str = "bfloat16"         # "float32": weights, activations and cache in fp32 (families that support it)
+    state_slots: int = 0            # recurrent-state slots (models with per-sequence state); 0: max_batch
 
     @classmethod
     def from_settings(cls, s) -> "EngineOptions":
@@ -66,7 +67,7 @@ def build_engine(opts: EngineOptions, comm=None, metrics=None) -> LLMEngine:
     dev = torch.device(opts.device)
     if dev.type == "cuda":
         # fail loudly: the GPU path never runs without the HIP kernels of the model's family
-        if getattr(cfg, "family", "llama") == "vivepel":
+        if getattr(cfg, "family", "llama") in ("vivepel", "kafilorn"):
             from ..ops._hip import require_mixers
             require_mixers()
         else:
@@ -78,7 +79,8 @@ def build_engine(opts: EngineOptions, comm=None, metrics=None) -> LLMEngine:
     dtype = torch.float32 if opts.dtype == "float32" else torch.bfloat16
     family = getattr(cfg, "family", "llama")
     if dtype == torch.float32 and family in ("llama", "mixtral"):
-        raise ValueError("the Llama / Mixtral kernels are bf16; float32 is served by the fp32-residual families (vivepel)")
+        raise ValueError("the Llama / Mixtral kernels are bf16; float32 is served by the fp32-residual families "
+                         "(vivepel, kafilorn)")
     if dtype == torch.float32:   # true fp32 products: no reduced-precision matrix mode
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False
@@ -127,7 +129,7 @@ def build_engine(opts: EngineOptions, comm=None, metrics=None) -> LLMEngine:
     runner = ModelRunner(cfg, weights, dev, num_blocks=num_blocks, block_size=opts.block_size,
                          max_model_len=opts.max_model_len, graph_buckets=opts.graph_buckets, mask_bits=masks,
                          comm=comm, tp_rank=opts.tp_rank, tp_size=opts.tp_size, ep_rank=par.ep_rank,
-                         ep_size=ep_size, use_graphs=opts.use_graphs)
+                         ep_size=ep_size, use_graphs=opts.use_graphs, num_state_slots=opts.state_slots or opts.max_batch)
     step_tokens = opts.max_batched_tokens if opts.max_batched_tokens > 0 else cfg.default_step_tokens()
     eng = LLMEngine(runner, tok, max_batch=opts.max_batch, max_batched_tokens=step_tokens,
                     max_model_len=opts.max_model_len, prefix_caching=opts.prefix_caching, metrics=metrics)

@@ -52,12 +52,15 @@ class LLMEngine:
                  max_model_len: int = 4096, prefix_caching: bool = True, metrics=None):
         self.runner = runner
         self.tokenizer = tokenizer
+        # prefix caching skips the cached tokens' forward: not for models whose recurrent state those tokens build
+        prefix_caching = prefix_caching and getattr(runner.model, "supports_prefix_cache", True)
         self.bm = make_block_manager(runner.num_blocks, runner.block_size, enable_prefix_caching=prefix_caching)
         self.scheduler = Scheduler(self.bm, max_batch=max_batch, max_batched_tokens=max_batched_tokens,
                                    max_model_len=max_model_len,
                                    partial_block_reuse=getattr(runner.model, "supports_block_copy", True),
                                    gather_max_s=float(os.environ.get("KA_GATHER_MAX_MS", "15")) / 1000.0,
-                                   gather_quiet_s=float(os.environ.get("KA_GATHER_QUIET_MS", "1.5")) / 1000.0)
+                                   gather_quiet_s=float(os.environ.get("KA_GATHER_QUIET_MS", "1.5")) / 1000.0,
+                                   state_slots=runner.state_slots)
         self.metrics = metrics
         self._inbox: "queue.SimpleQueue" = queue.SimpleQueue()
         self._wake = threading.Event()
@@ -195,8 +198,7 @@ class LLMEngine:
         seq.error = error
         seq.t_finish = time.perf_counter()
         self._live.pop(seq.seq_id, None)
-        if seq.block_table:
-            self.bm.free_table(seq.block_table)
+        self.scheduler.free_seq(seq)
         if seq.callback is not None:
             try:
                 seq.callback(seq)

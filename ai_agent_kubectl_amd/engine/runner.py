@@ -73,7 +73,7 @@ class ModelRunner:
     def __init__(self, cfg: ModelConfig, weights: Dict[str, torch.Tensor], device: torch.device,
                  num_blocks: int, block_size: int = 16, max_model_len: int = 4096, graph_buckets=(1, 2, 4, 8),
                  mask_bits: Optional[np.ndarray] = None, comm=None, tp_rank: int = 0, tp_size: int = 1,
-                 ep_rank: int = 0, ep_size: int = 1, use_graphs: bool = True):
+                 ep_rank: int = 0, ep_size: int = 1, use_graphs: bool = True, num_state_slots: int = 0):
         self.cfg = cfg
         self.device = torch.device(device)
         self.comm = comm or LocalComm()
@@ -93,6 +93,14 @@ class ModelRunner:
         self.num_blocks = num_blocks
         self.max_blocks = (max_model_len + block_size - 1) // block_size
         self.k_cache, self.v_cache = self.model.alloc_cache(num_blocks, block_size)
+        # models with per-sequence recurrent state own its tensors too (`alloc_state`); the slot pool is
+        # handed to the scheduler, which gives every admitted sequence one slot until it ends
+        self.state_slots = None
+        if hasattr(self.model, "alloc_state") and getattr(cfg, "has_state", False):
+            from .block_manager import StateSlots
+            n_slots = num_state_slots or max(int(b) for b in graph_buckets)
+            self.model.alloc_state(n_slots)
+            self.state_slots = StateSlots(n_slots)
         self.mask_bits = (torch.from_numpy(mask_bits.view(np.int32)).to(self.device)
                           if mask_bits is not None else None)
         self.buckets = sorted(set(int(b) for b in graph_buckets))
@@ -101,8 +109,9 @@ class ModelRunner:
         # ---- decode staging: [ids | pos | slots | ctx | mask | block_tables] at fixed offsets ----
         B = self.bmax
         # nsh: the leading block-table entries every row shares (cascade decode attention, 16-int slot)
-        self._off = {"ids": 0, "pos": B, "slots": 2 * B, "ctx": 3 * B, "mask": 4 * B, "nsh": 5 * B, "bt": 5 * B + 16}
-        self._stage_len = 5 * B + 16 + B * self.max_blocks
+        self._off = {"ids": 0, "pos": B, "slots": 2 * B, "ctx": 3 * B, "mask": 4 * B, "state": 5 * B, "nsh": 6 * B,
+                     "bt": 6 * B + 16}
+        self._stage_len = 6 * B + 16 + B * self.max_blocks
         # cascade decode attention from this bucket up (KA_CASCADE_MIN_B; 0 = off, the default): the
         # shared prefix blocks attended once per kv head and 16 query rows instead of once per row.
         # Measured slower at B = 64 / 256 with a 5-block shared prefix (+0.23 / +0.14 ms per step,
@@ -175,7 +184,8 @@ class ModelRunner:
         meta = AttnMeta(positions=self._view("pos", B), slot_mapping=self._view("slots", B),
                         block_tables=self._view("bt", B), ctx_lens=self._view("ctx", B),
                         logits_indices=self.d_logits_idx[:B], is_decode=True,
-                        shared_blocks=self._view("nsh", 1) if self._cascade(B) else None)
+                        shared_blocks=self._view("nsh", 1) if self._cascade(B) else None,
+                        state_slots=self._view("state", B) if self.state_slots is not None else None)
         return self.model.forward(self._view("ids", B), meta, self.k_cache, self.v_cache)
 
     def autotune(self) -> dict:
@@ -412,7 +422,7 @@ class ModelRunner:
             self.prefill_plan = self.tune_prefill()
         self.h_np[:] = 0
         o = self._off
-        for name in ("slots",):
+        for name in ("slots", "state"):
             self.h_np[o[name]:o[name] + self.bmax] = -1
         self.h_np[o["mask"]:o["mask"] + self.bmax] = -1
         self.d_stage.copy_(self.h_stage)
@@ -454,11 +464,12 @@ class ModelRunner:
             h[o["slots"] + i] = self._slot(s.block_table, pos)
             h[o["ctx"] + i] = L
             h[o["mask"] + i] = mask_index_for(s.num_generated + ahead, s.params.safe_decode)
+            h[o["state"] + i] = s.state_slot
             row = o["bt"] + i * mb
             n = len(s.block_table)
             h[row:row + n] = s.block_table
         if Bp > B:  # padding rows: no cache write, empty context
-            for name, val in (("ids", 0), ("pos", 0), ("slots", -1), ("ctx", 0), ("mask", -1)):
+            for name, val in (("ids", 0), ("pos", 0), ("slots", -1), ("ctx", 0), ("mask", -1), ("state", -1)):
                 h[o[name] + B:o[name] + Bp] = val
         h[o["nsh"]] = self._shared_prefix_blocks(batch, h, ahead) if self._cascade(Bp) else 0
 
@@ -680,7 +691,7 @@ class ModelRunner:
 
     def _pack_prefill(self, batch: Batch, pad: bool = False, with_fix: bool = False):
         """Packed step metadata [ids | pos | slots | q_starts | ctx | mask | logits idx | block tables |
-        copies (src, dst) | fixups (dst, src)].  with_fix: also returns the number of PLACEHOLDER
+        state slots | copies (src, dst) | fixups (dst, src)].  with_fix: also returns the number of PLACEHOLDER
         fixups (flat id position, in-flight row) appended at the end (their ids are packed as the
         placeholder and replaced on the device)."""
         S = len(batch.seqs)
@@ -696,7 +707,7 @@ class ModelRunner:
                     fix.append((q0 + nq - 1, s.ph_row))
                 q0 += nq
         nf = len(fix)
-        buf = np.zeros(3 * T + (S + 1) + 3 * S + S * mb + 2 * nc + 2 * nf, dtype=np.int32)
+        buf = np.zeros(3 * T + (S + 1) + 4 * S + S * mb + 2 * nc + 2 * nf, dtype=np.int32)
         if nf:
             fx = np.asarray(fix, dtype=np.int32)
             buf[len(buf) - 2 * nf:len(buf) - nf] = fx[:, 0]
@@ -713,7 +724,8 @@ class ModelRunner:
         ctx = buf[o:o + S]; o += S
         mask = buf[o:o + S]; o += S
         lidx = buf[o:o + S]; o += S
-        bt = buf[o:o + S * mb].reshape(S, mb)
+        bt = buf[o:o + S * mb].reshape(S, mb); o += S * mb
+        state = buf[o:o + S]
         # one Python pass collects per-sequence scalars, token slices and tables; the per-token
         # arrays are then built with a handful of vectorised numpy ops (was ~10 numpy calls per
         # sequence: ~2.7 ms of GPU-idle host time for a 256-request prefill)
@@ -737,6 +749,7 @@ class ModelRunner:
                 raise RuntimeError(f"prefill row {i} (seq {s.seq_id}) has no KV blocks")
             bt[i, :len(tbl)] = tbl
             mask[i] = mask_index_for(ng, s.params.safe_decode)
+            state[i] = s.state_slot
         n_real = int(nqs.sum())
         ends = np.cumsum(nqs)
         q_starts[0] = 0
@@ -770,10 +783,11 @@ class ModelRunner:
         ctx = buf[o:o + S]; o += S
         mask = buf[o:o + S]; o += S
         lidx = buf[o:o + S].long(); o += S
-        bt = buf[o:o + S * mb].view(S, mb)
+        bt = buf[o:o + S * mb].view(S, mb); o += S * mb
+        state = buf[o:o + S]
         meta = AttnMeta(positions=pos, slot_mapping=slots, block_tables=bt, ctx_lens=ctx, logits_indices=lidx,
                         is_decode=False, q_starts=q_starts, max_q_len=max_q, num_decode=nd,
-                        num_tokens=t_real or T)
+                        num_tokens=t_real or T, state_slots=state if self.state_slots is not None else None)
         return ids, meta, mask
 
     @torch.inference_mode()

@@ -25,7 +25,7 @@ import time
 from dataclasses import dataclass, field
 from typing import Deque, List, Optional
 
-from .block_manager import BlockManager, NoFreeBlocks
+from .block_manager import BlockManager, NoFreeBlocks, StateSlots
 from .sequence import Sequence, SeqStatus
 
 
@@ -49,7 +49,8 @@ class Scheduler:
                  prefill_max_wait_s: Optional[float] = None, prefill_min_frac: Optional[float] = None,
                  partial_block_reuse: bool = True, gather_max_s: float = 0.0, gather_quiet_s: float = 0.0015,
                  hold_steps: Optional[int] = None, hold_max_s: Optional[float] = None,
-                 chunked_prefill: Optional[bool] = None, min_chunk: int = 256):
+                 chunked_prefill: Optional[bool] = None, min_chunk: int = 256,
+                 state_slots: Optional[StateSlots] = None):
         # Prefill batching under continuous arrivals: a prefill step is an eager (non-graph) step,
         # so while sequences are decoding, new arrivals are admitted together — when at least
         # max(4, prefill_min_frac * running) are waiting or the oldest has waited
@@ -88,6 +89,8 @@ class Scheduler:
         self.hold_steps = hold_steps
         self.hold_max_s = hold_max_s
         self.bm = block_manager
+        # models with per-sequence recurrent state: a sequence holds one slot from admission to its end
+        self.state_slots = state_slots
         self.max_batch = max_batch
         self.max_batched_tokens = max_batched_tokens
         self.max_model_len = max_model_len
@@ -120,8 +123,15 @@ class Scheduler:
             self.running.remove(seq)
         if seq in self.prefilling:
             self.prefilling.remove(seq)
-        self.bm.free_table(seq.block_table)
+        self.free_seq(seq)
         seq.status = SeqStatus.ABORTED
+
+    def free_seq(self, seq: Sequence) -> None:
+        """Give back what a sequence holds: its pages and, for models with recurrent state, its state slot."""
+        self.bm.free_table(seq.block_table)
+        if self.state_slots is not None and seq.state_slot >= 0:
+            self.state_slots.release(seq.state_slot)
+        seq.state_slot = -1
 
     # ------------------------------------------------------------------------------------------
     def _admit(self, copies: List[tuple]):
@@ -144,6 +154,8 @@ class Scheduler:
         n_cont = len(admitted)     # continued chunk rows are already counted in n_busy
         while self.waiting and budget > 0 and n_busy + len(admitted) - n_cont < self.max_batch:
             seq = self.waiting[0]
+            if self.state_slots is not None and self.state_slots.num_free == 0:
+                break
             try:
                 table, cached, hashes = self.bm.allocate_prompt(seq.all_ids)
             except NoFreeBlocks:
@@ -163,6 +175,8 @@ class Scheduler:
                 copies.append((part[0], table[cached // self.bm.block_size]))
                 cached += part[1]
             self.waiting.popleft()
+            if self.state_slots is not None:
+                seq.state_slot = self.state_slots.acquire()
             seq.block_table, seq.block_hashes = table, hashes
             seq.num_computed = cached
             seq.num_cached_prompt = cached
@@ -281,6 +295,10 @@ class Scheduler:
         for seq, n in items:
             if n <= 0 or seq.num_computed + n > seq.total_len:
                 raise ValueError(f"seq {seq.seq_id}: {n} tokens from {seq.num_computed} of {seq.total_len}")
+            if self.state_slots is not None and seq.state_slot < 0:
+                if seq.num_computed:
+                    raise ValueError(f"seq {seq.seq_id}: its state slot was given back after {seq.num_computed} tokens")
+                seq.state_slot = self.state_slots.acquire()
             self.bm.ensure_capacity(seq.block_table, seq.num_computed + n)
             seq.status = SeqStatus.RUNNING
             (dec if n == 1 and seq.num_computed > 0 and seq.num_computed + 1 == seq.total_len else pre).append((seq, n))
@@ -290,14 +308,14 @@ class Scheduler:
                      prefill_seqs=[s for s, _ in pre])
 
     def release(self, seq: Sequence) -> None:
-        """Give a sequence's pages back (a request that ends outside `on_step_done`)."""
-        self.bm.free_table(seq.block_table)
+        """Give a sequence's pages and state slot back (a request that ends outside `on_step_done`)."""
+        self.free_seq(seq)
         seq.status = SeqStatus.FINISHED
 
     def _preempt(self, seq: Sequence) -> None:
         """Recompute-style preemption: drop the KV, requeue; re-admission prefills all_ids."""
         self.running.remove(seq)
-        self.bm.free_table(seq.block_table)
+        self.free_seq(seq)
         seq.block_hashes = []
         seq.num_computed = 0
         seq.status = SeqStatus.WAITING

@@ -40,6 +40,7 @@ class Sequence:
     output_ids: List[int] = field(default_factory=list)
     block_table: List[int] = field(default_factory=list)
     block_hashes: List[int] = field(default_factory=list)
+    state_slot: int = -1            # recurrent-state slot (models with per-sequence state), -1: none held
     num_computed: int = 0           # tokens whose KV is in the cache
     num_cached_prompt: int = 0      # prompt tokens served by the prefix cache
     n_forced: int = 0

@@ -10,7 +10,8 @@ entries and of `want`; after every step `done <step>` is printed.  Nothing is sa
 
 The replay drives the engine's own parts: `build_engine` (model registry, weight loading, cache
 pool), the scheduler's `schedule_given` (pages from the block manager, decode rows first) and the
-runner's `execute_logits` (the packing, cache and forward of `execute`).
+runner's `execute_logits` (the packing, cache and forward of `execute`).  A model with recurrent state gets
+`max_requests` state slots, taken at a request's first entry and given back at its end like its pages.
 """
 from __future__ import annotations
 
@@ -38,7 +39,8 @@ class TraceSession:
         opts = EngineOptions(model=model_dir, weights=model_dir, device=dev, dtype=dtype, block_size=bs,
                              kv_cache_tokens=tokens, max_model_len=tokens, max_batch=max_requests,
                              graph_buckets=tuple(b for b in (1, 2, 4, 8, 16) if b <= max_requests) or (1,),
-                             use_graphs=False, safe_decode=False, prefix_caching=False, ignore_eos=True)
+                             use_graphs=False, safe_decode=False, prefix_caching=False, ignore_eos=True,
+                             state_slots=max_requests)
         self.engine = build_engine(opts)
         self.runner = self.engine.runner
         self.sched = self.engine.scheduler

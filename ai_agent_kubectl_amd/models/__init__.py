@@ -9,4 +9,7 @@ def model_class(cfg):
     if family == "vivepel":
         from .vivepel import VivepelModel
         return VivepelModel
+    if family == "kafilorn":
+        from .kafilorn import KafilornModel
+        return KafilornModel
     raise ValueError(f"no model class for family {family!r}")

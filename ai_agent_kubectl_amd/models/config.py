@@ -179,8 +179,236 @@ def vivepel_uniform(name: str, layers: int, hidden: int, heads: int, kv_heads: i
     return VivepelConfig(name, vocab, hidden, 1e-6, groups, tuple(LayerSpec(spec, ff) for _ in range(layers)))
 
 
+# ------------------------------------------------------------------------------------------------
+# Kafilorn: layers listed one by one; a layer's mixer is an mLSTM (recurrent matrix memory, state slots)
+# or latent attention (a low-rank key/value latent in the paged cache, sliding window, softmax sink,
+# optionally borrowing another layer's cache); its feed-forward is dense (squared ReLU), a mixture of
+# gated experts with a group-limited router, or absent; the residual is `streams` hyper-connected copies.
+@dataclasses.dataclass(frozen=True)
+class MLSTMSpec:
+    """Matrix-memory recurrent mixer: per head a [dim, vdim] state, a normaliser [dim] and a running maximum."""
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float             # gate pre-activations pass through cap * tanh(. / cap); 0: uncapped
+    kind: str = "mlstm"
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "MLSTMSpec":
+        return cls(heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), gate_cap=float(m.get("gate_cap") or 0.0))
+
+    def to_dict(self) -> dict:
+        d = {"heads": self.heads, "dim": self.dim, "vdim": self.vdim}
+        if self.gate_cap:
+            d["gate_cap"] = self.gate_cap
+        return d
+
+    def state_floats(self) -> int:
+        return self.heads * (self.dim * self.vdim + self.dim + 1)
+
+
+@dataclasses.dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose keys and values are up-projections of a cached latent [kv_rank] plus one rotated key
+    part [rot_dim] shared by all heads; queries come through a latent of their own [q_rank]."""
+    heads: int
+    dim: int                    # unrotated query / key entries per head
+    rot_dim: int                # rotated query / key entries per head (the key part is shared by the heads)
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    window: int                 # position i sees j with 0 <= i - j < window (0: all of 0 .. i)
+    rot_dims: int               # rotary on the first rot_dims entries of the rotated part
+    rot_base: float
+    scale: float
+    kv_from: int = -1           # >= 0: no key/value down-projection of its own, reads that layer's cache
+    kind: str = "latent_attention"
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "LatentAttentionSpec":
+        mask, rot = m.get("mask"), m.get("rot")
+        kv_from = m.get("kv_from")
+        spec = cls(heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
+                   q_rank=int(m["q_rank"]), kv_rank=int(m["kv_rank"]), window=int(mask["size"]) if mask else 0,
+                   rot_dims=int(rot["dims"]) if rot else 0, rot_base=float(rot["base"]) if rot else 1.0,
+                   scale=float(m["scale"]), kv_from=-1 if kv_from is None else int(kv_from))
+        if spec.rot_dims % 2 or spec.rot_dims > spec.rot_dim or spec.window < 0:
+            raise ValueError(f"bad rotary dims {spec.rot_dims} / window {spec.window} for rotated size {spec.rot_dim}")
+        return spec
+
+    def to_dict(self) -> dict:
+        d = {"heads": self.heads, "dim": self.dim, "rot_dim": self.rot_dim, "vdim": self.vdim, "q_rank": self.q_rank,
+             "kv_rank": self.kv_rank, "scale": self.scale}
+        if self.window:
+            d["mask"] = {"size": self.window}
+        if self.rot_dims:
+            d["rot"] = {"base": self.rot_base, "dims": self.rot_dims}
+        if self.kv_from >= 0:
+            d["kv_from"] = self.kv_from
+        return d
+
+
+@dataclasses.dataclass(frozen=True)
+class FeedForwardSpec:
+    """dense: down(relu(up h)^2), width ff.  moe: `experts` gated experts of width ff, `top` per token chosen
+    among the best `keep_groups` of `groups` groups of neighbouring experts, plus a shared gated expert of
+    width shared_ff for every token (0: none)."""
+    kind: str                   # "dense" | "moe"
+    ff: int
+    experts: int = 0
+    top: int = 0
+    groups: int = 1
+    keep_groups: int = 1
+    shared_ff: int = 0
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "FeedForwardSpec":
+        if m["kind"] == "dense":
+            return cls("dense", int(m["ff"]))
+        if m["kind"] != "moe":
+            raise ValueError(f"unknown feed-forward kind {m['kind']!r}")
+        r, g, sh = m["router"], m["router"].get("groups"), m.get("shared")
+        spec = cls("moe", int(m["expert"]["ff"]), experts=int(r["experts"]), top=int(r["top"]),
+                   groups=int(g["count"]) if g else 1, keep_groups=int(g["keep"]) if g else 1,
+                   shared_ff=int(sh["ff"]) if sh else 0)
+        if spec.experts % spec.groups or not 0 < spec.keep_groups <= spec.groups or not 0 < spec.top <= spec.experts:
+            raise ValueError(f"bad router: {spec}")
+        if spec.top > spec.keep_groups * (spec.experts // spec.groups):
+            raise ValueError(f"router: top {spec.top} exceeds the experts of {spec.keep_groups} groups")
+        return spec
+
+    def to_dict(self) -> dict:
+        if self.kind == "dense":
+            return {"kind": "dense", "ff": self.ff}
+        r = {"experts": self.experts, "top": self.top}
+        if self.groups > 1:
+            r["groups"] = {"count": self.groups, "keep": self.keep_groups}
+        d = {"kind": "moe", "expert": {"ff": self.ff}, "router": r}
+        if self.shared_ff:
+            d["shared"] = {"ff": self.shared_ff}
+        return d
+
+
+@dataclasses.dataclass(frozen=True)
+class KafilornLayer:
+    mixer: object               # MLSTMSpec | LatentAttentionSpec
+    mlp: Optional[FeedForwardSpec]
+
+
+_KAFILORN_MIXERS = {"mlstm": MLSTMSpec, "latent_attention": LatentAttentionSpec}
+
+
+@dataclasses.dataclass(frozen=True)
+class KafilornConfig:
+    name: str
+    vocab_size: int
+    hidden: int
+    norm_eps: float
+    streams: int                # hyper-connection streams; 0: a plain residual sum
+    embed_scale: float
+    logit_scale: float
+    layers: Tuple[KafilornLayer, ...]
+    max_position: int = 1 << 20
+    tokenizer: str = "llama3"
+    family: str = "kafilorn"
+    tie_embeddings: bool = False
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return False            # its experts are not sharded: the engine's expert-parallel wiring does not apply
+
+    @property
+    def has_state(self) -> bool:
+        return any(L.mixer.kind == "mlstm" for L in self.layers)
+
+    @classmethod
+    def from_dict(cls, d: dict, name: str = "kafilorn") -> "KafilornConfig":
+        layers = []
+        for i, L in enumerate(d["layers"]):
+            if L["type"] not in _KAFILORN_MIXERS:
+                raise ValueError(f"layer {i}: unknown mixer type {L['type']!r}")
+            mixer = _KAFILORN_MIXERS[L["type"]].from_dict(L["mixer"])
+            layers.append(KafilornLayer(mixer, FeedForwardSpec.from_dict(L["mlp"]) if L.get("mlp") is not None else None))
+        for i, L in enumerate(layers):
+            m = L.mixer
+            if m.kind == "latent_attention" and m.kv_from >= 0:
+                src = layers[m.kv_from].mixer if 0 <= m.kv_from < i else None
+                if (src is None or src.kind != "latent_attention" or src.kv_from >= 0 or
+                        (src.kv_rank, src.rot_dim, src.rot_dims, src.rot_base) != (m.kv_rank, m.rot_dim, m.rot_dims, m.rot_base)):
+                    raise ValueError(f"layer {i}: kv_from {m.kv_from} must name an earlier latent-attention layer with "
+                                     "its own key/value latent of the same sizes and rotation")
+        emb = d.get("embedding") or {}
+        return cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]), norm_eps=float(d["norm"]["eps"]),
+                   streams=int(d.get("streams") or 0), embed_scale=float(emb.get("scale", 1.0)),
+                   logit_scale=float(d.get("logit_scale", 1.0)), layers=tuple(layers))
+
+    def to_dict(self) -> dict:
+        d = {"architecture": "Kafilorn", "vocab": self.vocab_size, "width": self.hidden, "norm": {"eps": self.norm_eps},
+             "embedding": {"scale": self.embed_scale}, "logit_scale": self.logit_scale,
+             "layers": [{"type": L.mixer.kind, "mixer": L.mixer.to_dict(), "mlp": L.mlp.to_dict() if L.mlp else None}
+                        for L in self.layers]}
+        if self.streams:
+            d["streams"] = self.streams
+        return d
+
+    def num_params(self) -> int:
+        h = self.hidden
+        n = 2 * self.vocab_size * h + h
+        for L in self.layers:
+            m, f = L.mixer, L.mlp
+            if m.kind == "mlstm":
+                n += h * m.heads * (2 * m.dim + 3 * m.vdim + 2) + m.heads * (m.vdim + 2)
+            else:
+                n += h * m.q_rank + m.q_rank * (1 + m.heads * (m.dim + m.rot_dim)) + m.heads * (m.kv_rank * (m.dim + m.vdim) + m.vdim * h + 1)
+                if m.kv_from < 0:
+                    n += h * (m.kv_rank + m.rot_dim) + m.kv_rank
+            if f is not None:
+                n += 2 * h * f.ff if f.kind == "dense" else 3 * h * (f.ff * f.experts + f.shared_ff) + f.experts * (h + 1)
+            n += 2 * h + 2 * (2 * self.streams + self.streams ** 2)
+        return n
+
+    def default_step_tokens(self) -> int:
+        return 8192
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        """Paged cache per token: the latent and the shared rotated key part of every layer that owns them."""
+        return max(1, sum((L.mixer.kv_rank + L.mixer.rot_dim) * dtype_bytes for L in self.layers
+                          if L.mixer.kind == "latent_attention" and L.mixer.kv_from < 0))
+
+    def state_bytes_per_slot(self) -> int:
+        """Recurrent state per sequence slot (fp32 in every engine dtype)."""
+        return sum(L.mixer.state_floats() * 4 for L in self.layers if L.mixer.kind == "mlstm")
+
+
+def kafilorn_uniform(name: str, blocks: int, hidden: int, heads: int, vocab: int, ff: int, experts: int = 8, top: int = 2,
+                     expert_ff: int = 0, window: int = 1024, streams: int = 2, kv_rank: int = 0, q_rank: int = 0,
+                     dim: int = 0, rot_dim: int = 0) -> KafilornConfig:
+    """`blocks` repetitions of (mLSTM + dense, latent attention + experts, latent attention on the previous layer's
+    cache + dense): a regular Kafilorn of given width (benchmarks, tests)."""
+    dim = dim or hidden // heads
+    rot_dim = rot_dim or dim // 2
+    ml = MLSTMSpec(heads, dim, dim, 15.0)
+    dense = FeedForwardSpec("dense", ff)
+    groups = next(g for g in (4, 3, 2, 1) if experts % g == 0)
+    keep = next(k for k in range(max(1, groups // 2), groups + 1) if k * (experts // groups) >= top)
+    moe = FeedForwardSpec("moe", expert_ff or ff // 4, experts=experts, top=top, groups=groups, keep_groups=keep,
+                          shared_ff=expert_ff or ff // 4)
+    layers = []
+    for b in range(blocks):
+        own = 3 * b + 1
+        att = dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=dim, q_rank=q_rank or hidden // 2, kv_rank=kv_rank or hidden // 4,
+                   window=window, rot_dims=rot_dim, rot_base=10000.0, scale=(dim + rot_dim) ** -0.5)
+        layers += [KafilornLayer(ml, dense), KafilornLayer(LatentAttentionSpec(**att), moe),
+                   KafilornLayer(LatentAttentionSpec(**att, kv_from=own), dense)]
+    return KafilornConfig(name, vocab, hidden, 1e-6, streams, 1.0, 1.0, tuple(layers))
+
+
 # config.json "architecture" -> parser of the file's dict
-ARCHITECTURES = {"Vivepel": VivepelConfig.from_dict}
+ARCHITECTURES = {"Vivepel": VivepelConfig.from_dict, "Kafilorn": KafilornConfig.from_dict}
 
 
 def load_config_dir(path: str):
@@ -218,6 +446,11 @@ PRESETS: Dict[str, ModelConfig] = {
     "tiny-vivepel": vivepel_uniform("tiny-vivepel", 2, 128, 4, 2, 32, 192, 384, chunk=16, rot_dims=12, groups=2),
     "vivepel-8b-2l": vivepel_uniform("vivepel-8b-2l", 2, 4096, 32, 8, 128, 14336, 128256),
     "vivepel-8b": vivepel_uniform("vivepel-8b", 32, 4096, 32, 8, 128, 14336, 128256),
+    # Kafilorn at a small size (CPU tests) and at a Llama-3-8B-like width (bench.py --arch-compare)
+    "tiny-kafilorn": kafilorn_uniform("tiny-kafilorn", 1, 128, 4, 384, 256, experts=6, top=2, expert_ff=64, window=24,
+                                      streams=2, kv_rank=48, q_rank=40, dim=24, rot_dim=8),
+    "kafilorn-4k-3l": kafilorn_uniform("kafilorn-4k-3l", 1, 4096, 32, 128256, 14336, experts=8, top=2, expert_ff=3584,
+                                       window=1024, streams=2, kv_rank=512, q_rank=1536, dim=128, rot_dim=64),
 }
 
 

@@ -50,6 +50,7 @@ class AttnMeta:
     num_decode: int = 0                # mixed step: the first num_decode sequences are 1-token decode rows
     num_tokens: int = 0                # real tokens when the step is padded (rows beyond are padding)
     shared_blocks: Optional[torch.Tensor] = None   # decode: [1] leading blocks shared by every row (cascade)
+    state_slots: Optional[torch.Tensor] = None     # [S] recurrent-state slot of each sequence (-1: padding row)
 
 
 class LlamaModel:

@@ -308,6 +308,180 @@ def load_vivepel_safetensors(path: str, cfg, device="cpu", dtype=torch.bfloat16)
     return W
 
 
+# ------------------------------------------------------------------------------------------------
+# Kafilorn.  Engine layout per layer `layers.<i>.` (activation dtype unless marked fp32):
+#   norm1, norm2, hc{1,2}_in [S], hc{1,2}_out [S], hc{1,2}_mix [S, S]                         fp32
+#   mLSTM:  w_proj [q; k; v; g rows, W] (one GEMM), w_if [2H, W] + b_if [2H] fp32 (input gates, then forget
+#           gates), hnorm [H * Dv] fp32, wo [W, H * Dv]
+#   latent attention:  w_dn [dq rows; dkv rows, W] (one GEMM; dq alone when the layer borrows another layer's
+#           cache), q_norm [Q] / kv_norm [R] / sink [H] / inv_freq fp32, w_uq [H * (D + Dr), Q],
+#           w_uk [H, D, R], w_uv [H, Dv, R], wo [W, H * Dv]
+#   dense feed-forward:  w_up [ff, W], w_down [W, ff]
+#   experts:  w_router [E, W] + correction [E] fp32, w_gu [E, 2 ff, W] (gate rows, then up rows),
+#           w_dn_e [E, W, ff], shared expert ws_gu [2 sff, W], ws_down [W, sff]
+# A model without streams is stored with S = 1 and unit stream weights (the plain residual sum).
+_KAFILORN_F32 = ("norm1", "norm2", "hc1_in", "hc1_out", "hc1_mix", "hc2_in", "hc2_out", "hc2_mix", "w_if", "b_if", "hnorm",
+                 "q_norm", "kv_norm", "sink", "inv_freq", "w_router", "correction")
+
+
+def _kafilorn_pack(cfg, get, device, dtype) -> Dict[str, torch.Tensor]:
+    S = max(cfg.streams, 1)
+    W: Dict[str, torch.Tensor] = {"embed": get("embed"), "lm_head": get("head"), "norm": get("final.norm").float(),
+                                  "ones": torch.ones(S)}
+    for i, L in enumerate(cfg.layers):
+        p, c, m, f = f"layers.{i}.", f"l{i}.", L.mixer, L.mlp
+        for q in ("1", "2") if f is not None else ("1",):
+            W[p + "norm" + q] = get(c + "norm" + q)
+            for k in ("in", "out", "mix"):
+                W[p + f"hc{q}_{k}"] = get(c + f"hc{q}.{k}") if cfg.streams else torch.ones((1, 1) if k == "mix" else (1,))
+        if m.kind == "mlstm":
+            W[p + "w_proj"] = torch.cat([get(c + "mix.q"), get(c + "mix.k"), get(c + "mix.v"), get(c + "mix.g")])
+            W[p + "w_if"] = torch.cat([get(c + "mix.i"), get(c + "mix.f")])
+            W[p + "b_if"] = torch.cat([get(c + "mix.i.b"), get(c + "mix.f.b")])
+            W[p + "hnorm"], W[p + "wo"] = get(c + "mix.norm"), get(c + "mix.o")
+        else:
+            own = m.kv_from < 0
+            W[p + "w_dn"] = torch.cat([get(c + "mix.dq"), get(c + "mix.dkv")]) if own else get(c + "mix.dq")
+            W[p + "q_norm"] = get(c + "mix.dq.norm")
+            if own:
+                W[p + "kv_norm"] = get(c + "mix.dkv.norm")
+            W[p + "w_uq"] = get(c + "mix.uq")
+            W[p + "w_uk"] = get(c + "mix.uk").view(m.heads, m.dim, m.kv_rank)
+            W[p + "w_uv"] = get(c + "mix.uv").view(m.heads, m.vdim, m.kv_rank)
+            W[p + "sink"], W[p + "wo"] = get(c + "mix.sink"), get(c + "mix.o")
+            half = m.rot_dims // 2
+            # base^(-2i / dims) in float64, rounded once to fp32; the angle is position * inv_freq in fp32
+            W[p + "inv_freq"] = float(m.rot_base) ** (-2.0 * torch.arange(half, dtype=torch.float64) / max(m.rot_dims, 1))
+        if f is None:
+            continue
+        if f.kind == "dense":
+            W[p + "w_up"], W[p + "w_down"] = get(c + "mlp.up"), get(c + "mlp.down")
+        else:
+            W[p + "w_router"], W[p + "correction"] = get(c + "mlp.router"), get(c + "mlp.correction")
+            W[p + "w_gu"] = torch.stack([torch.cat([get(c + f"mlp.e{e}.gate"), get(c + f"mlp.e{e}.up")]) for e in range(f.experts)])
+            W[p + "w_dn_e"] = torch.stack([get(c + f"mlp.e{e}.down") for e in range(f.experts)])
+            if f.shared_ff:
+                W[p + "ws_gu"] = torch.cat([get(c + "mlp.shared.gate"), get(c + "mlp.shared.up")])
+                W[p + "ws_down"] = get(c + "mlp.shared.down")
+    out = {}
+    for k, v in W.items():
+        f32 = k in ("norm", "ones") or k.rsplit(".", 1)[-1] in _KAFILORN_F32
+        out[k] = v.to(device=device, dtype=torch.float32 if f32 else dtype).contiguous()
+    return out
+
+
+def kafilorn_check_shapes(cfg, W: Dict[str, torch.Tensor]) -> None:
+    """Every tensor of the engine layout has the shape the configuration implies."""
+    h, V, S = cfg.hidden, cfg.vocab_size, max(cfg.streams, 1)
+    want = {"embed": (V, h), "lm_head": (V, h), "norm": (h,)}
+    for i, L in enumerate(cfg.layers):
+        p, m, f = f"layers.{i}.", L.mixer, L.mlp
+        for q in ("1", "2") if f is not None else ("1",):
+            want.update({p + "norm" + q: (h,), p + f"hc{q}_in": (S,), p + f"hc{q}_out": (S,), p + f"hc{q}_mix": (S, S)})
+        if m.kind == "mlstm":
+            want.update({p + "w_proj": (2 * m.heads * (m.dim + m.vdim), h), p + "w_if": (2 * m.heads, h),
+                         p + "b_if": (2 * m.heads,), p + "hnorm": (m.heads * m.vdim,), p + "wo": (h, m.heads * m.vdim)})
+        else:
+            own = m.kv_from < 0
+            want.update({p + "w_dn": (m.q_rank + (m.kv_rank + m.rot_dim if own else 0), h), p + "q_norm": (m.q_rank,),
+                         p + "w_uq": (m.heads * (m.dim + m.rot_dim), m.q_rank), p + "w_uk": (m.heads, m.dim, m.kv_rank),
+                         p + "w_uv": (m.heads, m.vdim, m.kv_rank), p + "sink": (m.heads,), p + "wo": (h, m.heads * m.vdim),
+                         p + "inv_freq": (m.rot_dims // 2,)})
+            if own:
+                want[p + "kv_norm"] = (m.kv_rank,)
+        if f is not None and f.kind == "dense":
+            want.update({p + "w_up": (f.ff, h), p + "w_down": (h, f.ff)})
+        elif f is not None:
+            want.update({p + "w_router": (f.experts, h), p + "correction": (f.experts,), p + "w_gu": (f.experts, 2 * f.ff, h),
+                         p + "w_dn_e": (f.experts, h, f.ff)})
+            if f.shared_ff:
+                want.update({p + "ws_gu": (2 * f.shared_ff, h), p + "ws_down": (h, f.shared_ff)})
+    for k, shp in want.items():
+        if k not in W or tuple(W[k].shape) != shp:
+            raise ValueError(f"tensor {k}: expected shape {shp}, found {tuple(W[k].shape) if k in W else None}")
+
+
+def kafilorn_checkpoint_tensors(cfg, seed: int = 0, dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Random tensors under the checkpoint's own names (what a Kafilorn model.safetensors holds)."""
+    g = torch.Generator().manual_seed(_seed(seed, "kafilorn") & 0x7FFFFFFF)
+    h, V, S = cfg.hidden, cfg.vocab_size, cfg.streams
+
+    def mat(o, i, std=None):
+        return (torch.randn(o, i, generator=g) * (std if std is not None else i ** -0.5)).to(dtype)
+
+    def vec(n, lo=0.75, hi=1.25):
+        return (lo + (hi - lo) * torch.rand(n, generator=g)).to(dtype)
+
+    T = {"embed": mat(V, h, 1.0), "head": mat(V, h), "final.norm": vec(h)}
+    for i, L in enumerate(cfg.layers):
+        c, m, f = f"l{i}.", L.mixer, L.mlp
+        for q in ("1", "2") if f is not None else ("1",):
+            T[c + "norm" + q] = vec(h)
+            if S:
+                T[c + f"hc{q}.in"] = vec(S, 0.5 / S, 1.5 / S)
+                T[c + f"hc{q}.out"] = vec(S, 0.5, 1.0)
+                T[c + f"hc{q}.mix"] = (torch.eye(S) * 0.8 + torch.rand(S, S, generator=g) * (0.2 / S)).to(dtype)
+        if m.kind == "mlstm":
+            for k, n in (("q", m.dim), ("k", m.dim), ("v", m.vdim), ("g", m.vdim)):
+                T[c + "mix." + k] = mat(m.heads * n, h)
+            T[c + "mix.i"], T[c + "mix.f"] = mat(m.heads, h), mat(m.heads, h)
+            T[c + "mix.i.b"] = (torch.randn(m.heads, generator=g) * 0.5).to(dtype)
+            T[c + "mix.f.b"] = (3.0 + torch.randn(m.heads, generator=g)).to(dtype)
+            T[c + "mix.norm"], T[c + "mix.o"] = vec(m.heads * m.vdim), mat(h, m.heads * m.vdim)
+        else:
+            T[c + "mix.dq"], T[c + "mix.dq.norm"] = mat(m.q_rank, h), vec(m.q_rank)
+            T[c + "mix.uq"] = mat(m.heads * (m.dim + m.rot_dim), m.q_rank)
+            if m.kv_from < 0:
+                T[c + "mix.dkv"], T[c + "mix.dkv.norm"] = mat(m.kv_rank + m.rot_dim, h), vec(m.kv_rank)
+            T[c + "mix.uk"], T[c + "mix.uv"] = mat(m.heads * m.dim, m.kv_rank), mat(m.heads * m.vdim, m.kv_rank)
+            T[c + "mix.sink"] = torch.randn(m.heads, generator=g).to(dtype)
+            T[c + "mix.o"] = mat(h, m.heads * m.vdim)
+        if f is not None and f.kind == "dense":
+            T[c + "mlp.up"], T[c + "mlp.down"] = mat(f.ff, h), mat(h, f.ff)
+        elif f is not None:
+            T[c + "mlp.router"] = mat(f.experts, h, 2.0 * h ** -0.5)
+            T[c + "mlp.correction"] = (torch.randn(f.experts, generator=g) * (0.5 / f.experts)).to(dtype)
+            for e in list(range(f.experts)) + (["shared"] if f.shared_ff else []):
+                n, ff = (f"mlp.e{e}.", f.ff) if e != "shared" else ("mlp.shared.", f.shared_ff)
+                T[c + n + "gate"], T[c + n + "up"], T[c + n + "down"] = mat(ff, h), mat(ff, h), mat(h, ff)
+    return T
+
+
+def kafilorn_random_weights(cfg, seed: int = 0, device="cpu", dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Random-init Kafilorn weights: drawn in bf16 (as a checkpoint stores them), packed for `dtype`."""
+    T = kafilorn_checkpoint_tensors(cfg, seed)
+    W = _kafilorn_pack(cfg, T.__getitem__, device, dtype)
+    kafilorn_check_shapes(cfg, W)
+    return W
+
+
+def _safetensors_getter(path: str):
+    from safetensors import safe_open
+
+    files = [path] if os.path.isfile(path) else sorted(glob.glob(os.path.join(path, "*.safetensors")))
+    if not files:
+        raise FileNotFoundError(f"no .safetensors under {path}")
+    index = {}
+    for f in files:
+        hnd = safe_open(f, framework="pt", device="cpu")
+        for k in hnd.keys():
+            index[k] = hnd
+
+    def get(name):
+        if name not in index:
+            raise KeyError(f"{path}: tensor {name!r} is missing")
+        return index[name].get_tensor(name)
+
+    return get
+
+
+def load_kafilorn_safetensors(path: str, cfg, device="cpu", dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """A Kafilorn checkpoint (a file, or a folder holding model.safetensors / *.safetensors)."""
+    W = _kafilorn_pack(cfg, _safetensors_getter(path), device, dtype)
+    kafilorn_check_shapes(cfg, W)
+    return W
+
+
 def build_weights(spec: str, cfg: ModelConfig, par: ParallelInfo, device="cpu", dtype=torch.bfloat16):
     if getattr(cfg, "family", "") == "vivepel":
         if par.tp_size != 1 or par.ep_size != 1:
@@ -316,6 +490,13 @@ def build_weights(spec: str, cfg: ModelConfig, par: ParallelInfo, device="cpu", 
             seed = int(spec.split(":", 1)[1]) if ":" in spec else 0
             return vivepel_random_weights(cfg, seed=seed, device=device, dtype=dtype)
         return load_vivepel_safetensors(spec, cfg, device=device, dtype=dtype)
+    if getattr(cfg, "family", "") == "kafilorn":
+        if par.tp_size != 1 or par.ep_size != 1:
+            raise ValueError("Kafilorn runs at TP = 1 (data parallel replicas scale it out)")
+        if spec.startswith("random"):
+            seed = int(spec.split(":", 1)[1]) if ":" in spec else 0
+            return kafilorn_random_weights(cfg, seed=seed, device=device, dtype=dtype)
+        return load_kafilorn_safetensors(spec, cfg, device=device, dtype=dtype)
     if spec.startswith("random"):
         seed = int(spec.split(":", 1)[1]) if ":" in spec else 0
         return random_weights(cfg, par, seed=seed, device=device, dtype=dtype)

@@ -115,6 +115,19 @@ _MIX_SIGS = {
     "ka_chunk_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, F, I, P],
     "ka_chunk_attention_tile_ok": [I, I, I, I, I],
     "ka_chunk_attention_tile": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, F, P],
+    "ka_embed_streams": [P, P, P, I, I, I, F, I, I, P],
+    "ka_stream_norm": [P, P, P, P, I, I, I, F, I, P],
+    "ka_stream_update": [P, P, P, P, P, P, P, I, I, I, F, I, I, P],
+    "ka_relu_sq": [P, P, ctypes.c_long, I, P],
+    "ka_silu_mul_rows": [P, P, I, I, I, P],
+    "ka_headnorm_gate": [P, P, P, I, I, P, I, I, I, F, I, P],
+    "ka_mlstm_gates": [P, P, P, P, I, I, I, F, I, P],
+    "ka_mlstm_scan": [P, P, I, I, I, I, P, P, P, P, P, P, I, P, I, I, I, F, I, P],
+    "ka_latent_prep": [P, P, I, I, I, I, I, P, P, P, P, P, P, I, F, I, P],
+    "ka_rope_split_q": [P, P, P, P, P, I, I, I, I, I, I, P],
+    "ka_window_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P],
+    "ka_moe_route": [P, P, P, P, P, I, I, I, I, I, I, I, P],
+    "ka_moe_rows": [P, P, P, P, P, P, P, I, I, I, I, I, P],
 }
 MIXERS_LIB = os.path.join(LIB_DIR, "libkagent_mixers.so")
 _mix: Optional[ctypes.CDLL] = None

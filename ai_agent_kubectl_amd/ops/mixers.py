@@ -1,6 +1,8 @@
-"""Ops of the models that keep their residual stream in fp32 (`models/vivepel.py`): grouped RMS norm,
+"""Ops of the models that keep their residual stream in fp32.  `models/vivepel.py`: grouped RMS norm,
 post-norm + layer scale + residual add, PolyNorm, per-head norm + partial rotary + cache append, and
-attention with a chunked mask, soft-capped scores, a sink and head mixing.
+attention with a chunked mask, soft-capped scores, a sink and head mixing.  `models/kafilorn.py`: residual
+streams (hyper-connections) with LayerNorm, the mLSTM gates and recurrence over state slots, latent attention
+with a sliding window and a learned sink, squared ReLU, and expert routing in groups with a choice correction.
 
 Dispatch follows `ops/__init__.py`: a GPU tensor goes to the HIP kernel (`csrc/norms_f32.hip`,
 `csrc/attention_chunk.hip`, built into `ops/lib/libkagent_mixers.so`) and raises if that library is
@@ -12,6 +14,7 @@ from __future__ import annotations
 from typing import Optional
 
 import torch
+import torch.nn.functional as F
 
 from . import reference as ref
 from ._hip import check, require_mixers
@@ -159,4 +162,247 @@ def chunk_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                  block_tables.shape[0], _p(positions), _p(slots), _p(mix), T, H, G, D, Dv, int(chunk), BS,
                                  block_tables.shape[1], int(bool(sink)), float(scale), float(cap), _f32(q), _stream()),
           "chunk_attention")
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+# residual streams, mLSTM, latent attention, grouped routing (csrc/streams_f32.hip, mlstm.hip,
+# attention_latent.hip, moe_route.hip)
+MOE_ROWS_MAX = 64    # token x expert rows served by the matrix-vector expert kernels (decode steps); more: sorted GEMMs
+
+
+def embed_streams(ids: torch.Tensor, table: torch.Tensor, scale: float, streams: int) -> torch.Tensor:
+    """table[ids] * scale as fp32 in `streams` copies: the start of the residual streams [T, S, W]."""
+    if _ref(table):
+        return ref.embed_streams(ids, table, scale, streams)
+    lib = require_mixers()
+    T, (V, W) = ids.shape[0], table.shape
+    assert ids.dtype == torch.int32 and table.is_contiguous() and streams >= 1
+    out = torch.empty((T, streams, W), dtype=torch.float32, device=table.device)
+    check(lib.ka_embed_streams(_p(out), _p(table), _p(ids), T, W, V, float(scale), streams, _f32(table), _stream()),
+          "embed_streams")
+    return out
+
+
+def stream_norm(x: torch.Tensor, w_in: torch.Tensor, w: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+    """LayerNorm (weight, no bias) of sum_s w_in[s] x[:, s]: [T, S, W] fp32 -> [T, W] in out_dtype."""
+    if _ref(x):
+        return ref.stream_norm(x, w_in, w, eps, out_dtype)
+    lib = require_mixers()
+    T, S, W = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous() and w_in.dtype == torch.float32 and w_in.numel() == S
+    assert w.dtype == torch.float32 and w.numel() == W
+    out = torch.empty((T, W), dtype=out_dtype, device=x.device)
+    check(lib.ka_stream_norm(_p(out), _p(x), _p(w_in), _p(w), T, W, S, float(eps), _f32(out), _stream()), "stream_norm")
+    return out
+
+
+def stream_update(x: torch.Tensor, y: torch.Tensor, mix: torch.Tensor, out: torch.Tensor,
+                  next_in: Optional[torch.Tensor], next_w: Optional[torch.Tensor], eps: float, out_dtype):
+    """x[:, r] <- sum_s mix[s, r] x[:, s] + out[r] * y, in place; returns stream_norm(x, next_in, next_w) computed
+    in the same pass (None without next_w)."""
+    if _ref(x):
+        return ref.stream_update(x, y, mix, out, next_in, next_w, eps, out_dtype)
+    lib = require_mixers()
+    T, S, W = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous() and y.shape == (T, W) and y.is_contiguous()
+    assert mix.dtype == torch.float32 and mix.shape == (S, S) and mix.is_contiguous() and out.dtype == torch.float32
+    assert out.numel() == S and (next_w is None or (next_w.dtype == torch.float32 and next_w.numel() == W
+                                                     and next_in.dtype == torch.float32 and next_in.numel() == S))
+    h = torch.empty((T, W), dtype=out_dtype, device=x.device) if next_w is not None else None
+    check(lib.ka_stream_update(_p(x), _p(y), _p(mix), _p(out), _p(next_in) if next_w is not None else None, _p(next_w),
+                               _p(h), T, W, S, float(eps), _f32(y), _f32(h) if h is not None else 0, _stream()),
+          "stream_update")
+    return h
+
+
+def relu_sq(z: torch.Tensor) -> torch.Tensor:
+    """relu(z)^2, elementwise."""
+    if _ref(z):
+        return ref.relu_sq(z)
+    lib = require_mixers()
+    assert z.is_contiguous()
+    out = torch.empty_like(z)
+    check(lib.ka_relu_sq(_p(out), _p(z), z.numel(), _f32(z), _stream()), "relu_sq")
+    return out
+
+
+def silu_mul(gu: torch.Tensor) -> torch.Tensor:
+    """[T, 2 ff] = gate | up -> silu(gate) * up [T, ff] (bf16 or fp32)."""
+    if _ref(gu):
+        return ref.silu_mul(gu)
+    lib = require_mixers()
+    T, two = gu.shape
+    assert gu.is_contiguous() and two % 2 == 0
+    out = torch.empty((T, two // 2), dtype=gu.dtype, device=gu.device)
+    check(lib.ka_silu_mul_rows(_p(out), _p(gu), T, two // 2, _f32(gu), _stream()), "silu_mul_rows")
+    return out
+
+
+def mlstm_gates(h: torch.Tensor, w_if: torch.Tensor, b_if: torch.Tensor, cap: float) -> torch.Tensor:
+    """[T, 2H] fp32: log input gates (soft-capped), then log forget gates logsigmoid(soft-capped)."""
+    if _ref(h):
+        return ref.mlstm_gates(h, w_if, b_if, cap)
+    lib = require_mixers()
+    T, W = h.shape
+    assert h.is_contiguous() and w_if.dtype == torch.float32 and w_if.shape[1] == W and w_if.is_contiguous()
+    assert b_if.dtype == torch.float32 and b_if.numel() == w_if.shape[0] and w_if.shape[0] % 2 == 0
+    out = torch.empty((T, w_if.shape[0]), dtype=torch.float32, device=h.device)
+    check(lib.ka_mlstm_gates(_p(out), _p(h), _p(w_if), _p(b_if), T, W, w_if.shape[0] // 2, float(cap), _f32(h), _stream()),
+          "mlstm_gates")
+    return out
+
+
+def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gates: torch.Tensor, st_S: torch.Tensor,
+               st_n: torch.Tensor, st_m: torch.Tensor, seq_slots: torch.Tensor, q_starts: Optional[torch.Tensor],
+               positions: torch.Tensor, H: int, D: int, Dv: int, qscale: float) -> torch.Tensor:
+    """The mLSTM recurrence over each sequence's rows, from / into the state of its slot (st_S [slots, H, Dv, D],
+    st_n [slots, H, D], st_m [slots, H], fp32); a sequence whose first row is at position 0 starts from zero.
+    q_starts None: row t is sequence t.  -> [T, H * Dv] fp32 (numerator / denominator, before the head norm)."""
+    if _ref(proj):
+        S = st_S.transpose(-1, -2)
+        return ref.mlstm_scan(proj, q_off, k_off, v_off, gates, S, st_n, st_m, seq_slots, q_starts, positions, H, D, Dv,
+                              qscale)
+    lib = require_mixers()
+    T, P = proj.shape
+    nseq = seq_slots.shape[0]
+    assert proj.is_contiguous() and gates.dtype == torch.float32 and gates.shape == (T, 2 * H) and gates.is_contiguous()
+    assert max(q_off, k_off) + H * D <= P and v_off + H * Dv <= P
+    assert st_S.dtype == st_n.dtype == st_m.dtype == torch.float32 and st_S.shape[1:] == (H, Dv, D) and st_S.is_contiguous()
+    assert st_n.shape[1:] == (H, D) and st_m.shape[1:] == (H,) and st_n.is_contiguous() and st_m.is_contiguous()
+    assert seq_slots.dtype == torch.int32 and positions.dtype == torch.int32 and positions.shape[0] >= T
+    assert (q_starts is None and nseq <= T) or (q_starts is not None and q_starts.dtype == torch.int32
+                                                 and q_starts.shape[0] == nseq + 1)
+    out = torch.zeros((T, H * Dv), dtype=torch.float32, device=proj.device)
+    check(lib.ka_mlstm_scan(_p(out), _p(proj), P, q_off, k_off, v_off, _p(gates), _p(st_S), _p(st_n), _p(st_m),
+                            _p(seq_slots), _p(q_starts), nseq, _p(positions), H, D, Dv, float(qscale), _f32(proj),
+                            _stream()), "mlstm_scan")
+    return out
+
+
+def headnorm_gate(o: torch.Tensor, proj: torch.Tensor, g_off: int, w: torch.Tensor, H: int, Dv: int, eps: float,
+                  out_dtype) -> torch.Tensor:
+    """o [T, H * Dv] fp32: each head divided by its root mean square, times w, times sigmoid(proj[:, g_off:...])."""
+    if _ref(o):
+        return ref.headnorm_gate(o, proj, g_off, w, H, Dv, eps, out_dtype)
+    lib = require_mixers()
+    T = o.shape[0]
+    assert o.dtype == torch.float32 and o.is_contiguous() and proj.is_contiguous() and proj.dtype == out_dtype
+    assert g_off + H * Dv <= proj.shape[1] and w.dtype == torch.float32 and w.numel() == H * Dv
+    out = torch.empty((T, H * Dv), dtype=out_dtype, device=o.device)
+    check(lib.ka_headnorm_gate(_p(out), _p(o), _p(proj), proj.shape[1], g_off, _p(w), T, H, Dv, float(eps), _f32(out),
+                               _stream()), "headnorm_gate")
+    return out
+
+
+def latent_prep(proj: torch.Tensor, Q: int, R: int, Dr: int, w_q: torch.Tensor, w_kv: Optional[torch.Tensor],
+                inv_freq: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, cache: Optional[torch.Tensor],
+                rot_dims: int, eps: float) -> torch.Tensor:
+    """Rows [query latent Q | key/value latent R | rotated key part Dr] -> the RMS-normed query latent [T, Q];
+    with a cache [NB, BS, R + Dr], the normed latent and the rotated key part are appended at `slots`."""
+    if _ref(proj):
+        return ref.latent_prep(proj, Q, R, Dr, w_q, w_kv, inv_freq, positions, slots, cache, rot_dims, eps)
+    lib = require_mixers()
+    T, P = proj.shape
+    assert proj.is_contiguous() and w_q.dtype == torch.float32 and w_q.numel() == Q
+    assert positions.dtype == torch.int32 and slots.dtype == torch.int32 and positions.shape[0] >= T and slots.shape[0] >= T
+    if cache is not None:
+        assert cache.dtype == proj.dtype and cache.shape[2] == R + Dr and cache.is_contiguous() and P >= Q + R + Dr
+        assert w_kv.dtype == torch.float32 and w_kv.numel() == R and inv_freq.dtype == torch.float32
+        assert inv_freq.numel() * 2 == rot_dims
+    cq = torch.empty((T, Q), dtype=proj.dtype, device=proj.device)
+    check(lib.ka_latent_prep(_p(cq), _p(proj), T, P, Q, R, Dr, _p(w_q), _p(w_kv), _p(inv_freq), _p(positions), _p(slots),
+                             _p(cache), rot_dims, float(eps), _f32(proj), _stream()), "latent_prep")
+    return cq
+
+
+def rope_split_q(q: torch.Tensor, inv_freq: torch.Tensor, positions: torch.Tensor, H: int, D: int, Dr: int,
+                 rot_dims: int):
+    """q [T, H * (D + Dr)] -> (unrotated parts [H, T, D] in q's dtype, rotated parts after rotary [T, H, Dr] fp32)."""
+    if _ref(q):
+        return ref.rope_split_q(q, inv_freq, positions, H, D, Dr, rot_dims)
+    lib = require_mixers()
+    T = q.shape[0]
+    assert q.is_contiguous() and q.shape[1] == H * (D + Dr) and positions.dtype == torch.int32 and positions.shape[0] >= T
+    assert inv_freq.dtype == torch.float32 and inv_freq.numel() * 2 == rot_dims
+    qn = torch.empty((H, T, D), dtype=q.dtype, device=q.device)
+    qr = torch.empty((T, H, Dr), dtype=torch.float32, device=q.device)
+    check(lib.ka_rope_split_q(_p(qn), _p(qr), _p(q), _p(inv_freq), _p(positions), T, H, D, Dr, rot_dims, _f32(q), _stream()),
+          "rope_split_q")
+    return qn, qr
+
+
+def window_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor,
+                     q_starts: Optional[torch.Tensor], positions: torch.Tensor, slots: torch.Tensor,
+                     sink: Optional[torch.Tensor], window: int, scale: float) -> torch.Tensor:
+    """Multi-query attention over cache rows [latent R | rotated key part Dr] with the latent as the value:
+    q_lat [H, T, R], q_rot [T, H, Dr] fp32 -> [H, T, R].  window 0: all earlier keys; sink None: plain softmax."""
+    if _ref(q_lat):
+        return ref.window_attention(q_lat, q_rot, cache, block_tables, q_starts, positions, slots, sink, window, scale)
+    lib = require_mixers()
+    H, T, R = q_lat.shape
+    Dr, BS = q_rot.shape[2], cache.shape[1]
+    assert q_lat.is_contiguous() and q_rot.is_contiguous() and q_rot.dtype == torch.float32 and q_rot.shape[:2] == (T, H)
+    assert cache.dtype == q_lat.dtype and cache.is_contiguous() and cache.shape[2] == R + Dr
+    assert block_tables.dtype == torch.int32 and block_tables.is_contiguous() and block_tables.dim() == 2
+    assert positions.dtype == torch.int32 and slots.dtype == torch.int32 and positions.shape[0] >= T and slots.shape[0] >= T
+    assert q_starts is None or (q_starts.dtype == torch.int32 and q_starts.shape[0] == block_tables.shape[0] + 1)
+    assert q_starts is not None or block_tables.shape[0] >= T
+    assert sink is None or (sink.dtype == torch.float32 and sink.numel() == H)
+    out = torch.empty((H, T, R), dtype=q_lat.dtype, device=q_lat.device)
+    check(lib.ka_window_attention(_p(out), _p(q_lat), _p(q_rot), _p(cache), _p(block_tables), _p(q_starts),
+                                  block_tables.shape[0], _p(positions), _p(slots), _p(sink), T, H, R, Dr, BS,
+                                  block_tables.shape[1], int(window), float(scale), _f32(q_lat), _stream()),
+          "window_attention")
+    return out
+
+
+def moe_route(h: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int,
+              keep: int):
+    """-> (expert ids [T, top] int32, weights [T, top] fp32); see csrc/moe_route.hip."""
+    if _ref(h):
+        return ref.moe_route(h, w_router, correction, top, groups, keep)
+    lib = require_mixers()
+    T, W = h.shape
+    E = w_router.shape[0]
+    assert h.is_contiguous() and w_router.dtype == torch.float32 and w_router.shape[1] == W and w_router.is_contiguous()
+    assert correction is None or (correction.dtype == torch.float32 and correction.numel() == E)
+    ids = torch.empty((T, top), dtype=torch.int32, device=h.device)
+    w = torch.empty((T, top), dtype=torch.float32, device=h.device)
+    check(lib.ka_moe_route(_p(ids), _p(w), _p(h), _p(w_router), _p(correction), T, W, E, top, groups, keep, _f32(h),
+                           _stream()), "moe_route")
+    return ids, w
+
+
+def moe_experts(h: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """sum_k w[t, k] * expert_{ids[t, k]}(h[t]) -> [T, W] fp32; w_gu [E, 2 ff, W] (gate rows, then up rows),
+    w_down [E, W, ff].  A few rows (decode): matrix-vector kernels straight from the stacked weights, no host
+    read, capturable.  More: rows sorted by expert, one read of the per-expert counts, one vendor GEMM pair per
+    expert segment, weighted scatter-add in fp32."""
+    if _ref(h):
+        return ref.moe_experts(h, w_gu, w_down, ids, w)
+    T, W = h.shape
+    E, two_ff, _ = w_gu.shape
+    ff, top = two_ff // 2, ids.shape[1]
+    assert h.is_contiguous() and w_gu.is_contiguous() and w_down.is_contiguous() and w_gu.dtype == h.dtype == w_down.dtype
+    assert w_down.shape == (E, W, ff) and ids.dtype == torch.int32 and w.dtype == torch.float32 and w.shape == ids.shape
+    out = torch.zeros((T, W), dtype=torch.float32, device=h.device)
+    if T * top <= MOE_ROWS_MAX and W * 4 <= 60 * 1024 and top * ff * 4 <= 60 * 1024 and top <= 32:
+        lib = require_mixers()
+        act = torch.empty((T * top, ff), dtype=h.dtype, device=h.device)
+        check(lib.ka_moe_rows(_p(out), _p(act), _p(h), _p(w_gu), _p(w_down), _p(ids), _p(w), T, W, ff, top, _f32(h),
+                              _stream()), "moe_rows")
+        return out
+    flat = ids.reshape(-1).long()
+    order = torch.argsort(flat, stable=True)
+    counts = torch.bincount(flat, minlength=E).tolist()    # the layer's one host read (vendor GEMMs take host shapes)
+    tok = torch.div(order, top, rounding_mode="floor")
+    xs = h.index_select(0, tok)
+    ys = torch.empty((xs.shape[0], W), dtype=h.dtype, device=h.device)
+    off = 0
+    for e, c in enumerate(counts):
+        if c:
+            ys[off:off + c] = F.linear(silu_mul(F.linear(xs[off:off + c], w_gu[e])), w_down[e])
+            off += c
+    out.index_add_(0, tok, ys.float() * w.reshape(-1).index_select(0, order).unsqueeze(1))
     return out

@@ -236,3 +236,184 @@ def chunk_attention(q, k_cache, v_cache, block_tables, q_starts, positions, slot
         o = torch.einsum("hn,nhd->hd", w, v.repeat_interleave(rep, dim=1))
         out[t] = o.reshape(-1).to(q.dtype)
     return out
+
+
+# ------------------------------------------------------------------------------------------------
+# Stream (hyper-connection) residuals, mLSTM, latent attention with a window and a sink, grouped expert
+# routing (models/kafilorn.py): the ops of ops/mixers.py on CPU tensors, fp32 wherever the kernels are.
+def embed_streams(ids: torch.Tensor, table: torch.Tensor, scale: float, streams: int) -> torch.Tensor:
+    """table[ids] * scale as fp32, copied into `streams` residual streams: [T, S, W]."""
+    x = table[ids.long().clamp(0, table.shape[0] - 1)].float() * scale
+    return x[:, None, :].repeat(1, streams, 1).contiguous()
+
+
+def _layer_norm(u: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+    d = u - u.mean(-1, keepdim=True)
+    return d / torch.sqrt((d * d).mean(-1, keepdim=True) + eps) * w.float()
+
+
+def stream_norm(x: torch.Tensor, w_in: torch.Tensor, w: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+    """LayerNorm (weight, no bias) of u = sum_s w_in[s] x[:, s]."""
+    u = torch.einsum("tsw,s->tw", x, w_in.float())
+    return _layer_norm(u, w, eps).to(out_dtype)
+
+
+def stream_update(x, y, mix, out, next_in, next_w, eps: float, out_dtype):
+    """x[:, t] <- sum_s mix[s, t] x[:, s] + out[t] * y (in place, all streams from the old ones); returns
+    the next sublayer's normed input (stream_norm with next_in / next_w) or None."""
+    new = torch.einsum("tsw,sr->trw", x, mix.float()) + out.float()[None, :, None] * y.float()[:, None, :]
+    x.copy_(new)
+    return stream_norm(x, next_in, next_w, eps, out_dtype) if next_w is not None else None
+
+
+def relu_sq(z: torch.Tensor) -> torch.Tensor:
+    r = torch.relu(z.float())
+    return (r * r).to(z.dtype)
+
+
+def mlstm_gates(h: torch.Tensor, w_if: torch.Tensor, b_if: torch.Tensor, cap: float) -> torch.Tensor:
+    """[T, 2H] fp32: the capped log input gates, then the log forget gates logsigmoid(capped)."""
+    z = h.float() @ w_if.float().t() + b_if.float()
+    if cap > 0:
+        z = cap * torch.tanh(z / cap)
+    H = z.shape[1] // 2
+    return torch.cat([z[:, :H], F.logsigmoid(z[:, H:])], dim=1)
+
+
+def _seq_of(T: int, q_starts):
+    if q_starts is None:
+        return [(i, i, i + 1) for i in range(T)]
+    qs = q_starts.tolist()
+    return [(i, qs[i], qs[i + 1]) for i in range(len(qs) - 1)]
+
+
+def mlstm_scan(proj, q_off: int, k_off: int, v_off: int, gates, st_S, st_n, st_m, seq_slots, q_starts, positions,
+               H: int, D: int, Dv: int, qscale: float) -> torch.Tensor:
+    """The recurrence over each sequence's rows of this step, from the state in its slot (zero when the row's
+    position is 0) and back into it.  proj rows hold q [H, D], k [H, D], v [H, Dv] at the given column offsets.
+    -> num / den per head [T, H * Dv] fp32 (before the head norm)."""
+    T = proj.shape[0]
+    out = torch.zeros((T, H * Dv), dtype=torch.float32, device=proj.device)
+    slots, pos = seq_slots.tolist(), positions.tolist()
+    for i, a, b in _seq_of(T, q_starts):
+        sl = slots[i]
+        if sl < 0 or b <= a:
+            continue
+        if pos[a] == 0:
+            S, n, m = torch.zeros(H, D, Dv), torch.zeros(H, D), torch.zeros(H)
+        else:
+            S, n, m = st_S[sl].clone(), st_n[sl].clone(), st_m[sl].clone()
+        for t in range(a, b):
+            q = proj[t, q_off:q_off + H * D].float().view(H, D) * qscale
+            k = proj[t, k_off:k_off + H * D].float().view(H, D)
+            v = proj[t, v_off:v_off + H * Dv].float().view(H, Dv)
+            ig, fg = gates[t, :H], gates[t, H:]
+            m_new = torch.maximum(fg + m, ig)
+            fa, ia = torch.exp(fg + m - m_new), torch.exp(ig - m_new)
+            S = fa[:, None, None] * S + ia[:, None, None] * (k[:, :, None] * v[:, None, :])
+            n = fa[:, None] * n + ia[:, None] * k
+            m = m_new
+            den = torch.maximum((n * q).sum(-1).abs(), torch.exp(-m)) + 1e-6
+            out[t] = (torch.einsum("hdv,hd->hv", S, q) / den[:, None]).reshape(-1)
+        st_S[sl], st_n[sl], st_m[sl] = S, n, m
+    return out
+
+
+def headnorm_gate(o, proj, g_off: int, w, H: int, Dv: int, eps: float, out_dtype) -> torch.Tensor:
+    """Each head of o divided by its root mean square, times w, times sigmoid(gate columns of proj)."""
+    T = o.shape[0]
+    oh = o.view(T, H, Dv)
+    y = (oh / torch.sqrt((oh * oh).mean(-1, keepdim=True) + eps)).reshape(T, H * Dv) * w.float()
+    return (y * torch.sigmoid(proj[:, g_off:g_off + H * Dv].float())).to(out_dtype)
+
+
+def _rot(x, positions, inv_freq, dims: int):
+    half = dims // 2
+    if half == 0:
+        return x
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [half]
+    c, s = torch.cos(ang).view(shape), torch.sin(ang).view(shape)
+    a, b = x[..., :half], x[..., half:dims]
+    return torch.cat([a * c - b * s, b * c + a * s, x[..., dims:]], dim=-1)
+
+
+def latent_prep(proj, Q: int, R: int, Dr: int, w_q, w_kv, inv_freq, positions, slots, cache, rot_dims: int, eps: float):
+    """proj rows = [query latent Q | key/value latent R | rotated key part Dr] (the last two only with a cache).
+    -> the RMS-normed query latent [T, Q]; the normed latent and the rotated key part go to cache[slot]."""
+    cq = proj[:, :Q].float()
+    cq = (cq / torch.sqrt((cq * cq).mean(-1, keepdim=True) + eps) * w_q.float()).to(proj.dtype)
+    if cache is not None:
+        c = proj[:, Q:Q + R].float()
+        c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * w_kv.float()
+        kr = _rot(proj[:, Q + R:Q + R + Dr].float(), positions[:proj.shape[0]], inv_freq, rot_dims)
+        row = torch.cat([c, kr], dim=1).to(cache.dtype)
+        s = slots[:proj.shape[0]].long()
+        ok = s >= 0
+        if ok.any():
+            bs = cache.shape[1]
+            cache[s[ok] // bs, s[ok] % bs] = row[ok]
+    return cq.contiguous()
+
+
+def rope_split_q(q, inv_freq, positions, H: int, D: int, Dr: int, rot_dims: int):
+    """q [T, H * (D + Dr)] -> (unrotated parts [H, T, D] in q's dtype, rotated parts [T, H, Dr] fp32)."""
+    T = q.shape[0]
+    qh = q.view(T, H, D + Dr)
+    qn = qh[:, :, :D].transpose(0, 1).contiguous()
+    qr = _rot(qh[:, :, D:].float(), positions[:T], inv_freq, rot_dims).contiguous()
+    return qn, qr
+
+
+def window_attention(q_lat, q_rot, cache, block_tables, q_starts, positions, slots, sink, window: int, scale: float):
+    """One shared key [R + Dr] per token (multi-query): score = (q_lat . c + q_rot . k_rot) * scale over the
+    last `window` positions (0: all), softmax with an optional per-head sink logit in the denominator, values
+    = the latent c.  q_lat [H, T, R], q_rot [T, H, Dr] -> [H, T, R] in q_lat's dtype."""
+    H, T, R = q_lat.shape
+    bs = cache.shape[1]
+    out = torch.zeros((H, T, R), dtype=q_lat.dtype, device=q_lat.device)
+    pos_l, slot_l = positions.tolist(), slots.tolist()
+    for i, a, b in _seq_of(T, q_starts):
+        for t in range(a, b):
+            if slot_l[t] < 0:
+                continue
+            p = pos_l[t]
+            lo = max(0, p - window + 1) if window > 0 else 0
+            js = torch.arange(lo, p + 1)
+            rows = cache[block_tables[i].long()[js // bs], js % bs].float()       # [n, R + Dr]
+            s = (q_lat[:, t].float() @ rows[:, :R].t() + q_rot[t].float() @ rows[:, R:].t()) * scale
+            m = s.max(-1, keepdim=True).values
+            if sink is not None:
+                m = torch.maximum(m, sink.float()[:, None])
+            e = torch.exp(s - m)
+            den = e.sum(-1, keepdim=True) + (torch.exp(sink.float()[:, None] - m) if sink is not None else 0.0)
+            out[:, t] = ((e / den) @ rows[:, :R]).to(q_lat.dtype)
+    return out
+
+
+def moe_route(h, w_router, correction, top: int, groups: int, keep: int):
+    """Softmax scores over all experts; the choice adds `correction` and is limited to the `keep` groups (of
+    `groups` equal groups of neighbours) whose best choice score is largest; weights = the chosen experts'
+    scores (without correction) over their sum.  -> (ids [T, top] int32, weights [T, top] fp32)."""
+    s = torch.softmax(h.float() @ w_router.float().t(), dim=-1)
+    choice = s + correction.float() if correction is not None else s.clone()
+    T, E = s.shape
+    if groups > 1:
+        best = choice.view(T, groups, E // groups).max(-1).values
+        kept = torch.zeros_like(best, dtype=torch.bool).scatter_(1, torch.topk(best, keep, dim=-1).indices, True)
+        choice = choice.masked_fill(~kept.repeat_interleave(E // groups, dim=1), float("-inf"))
+    ids = torch.topk(choice, top, dim=-1).indices
+    w = s.gather(1, ids)
+    return ids.to(torch.int32), w / (w.sum(-1, keepdim=True) + 1e-20)
+
+
+def moe_experts(h, w_gu, w_down, ids, w) -> torch.Tensor:
+    """sum_k w[t, k] * down_e(silu(gate_e h) * up_e h), e = ids[t, k]; w_gu [E, 2 ff, W] = gate rows then up
+    rows, w_down [E, W, ff].  -> [T, W] fp32."""
+    T, W = h.shape
+    out = torch.zeros((T, W), dtype=torch.float32, device=h.device)
+    for e in torch.unique(ids).tolist():
+        tok, slot = torch.nonzero(ids == e, as_tuple=True)
+        y = F.linear(silu_mul(F.linear(h[tok], w_gu[e])), w_down[e])
+        out.index_add_(0, tok, y.float() * w[tok, slot][:, None])
+    return out
