@@ -15,7 +15,7 @@
 namespace {
 using namespace rows;
 
-constexpr int MAX_STREAMS = 8;
+constexpr int MAX_STREAMS = 16;
 
 template <typename AT>
 __global__ __launch_bounds__(NT) void embed_streams_kernel(float* __restrict__ out, const AT* __restrict__ table,

@@ -113,7 +113,10 @@ class SyntheticTokenizer:
                 words.append(p)
         n_fill = n_regular - byte_base - 256 - len(words)
         words += _pseudo_words(max(0, n_fill), seed, taken)
-        pieces += [w.encode("utf-8") for w in words[: n_regular - byte_base - 256]]
+        pieces += [w.encode("utf-8") for w in words[: max(0, n_regular - byte_base - 256)]]
+        # a vocabulary smaller than the byte table (checkpoints of test size, served by token ids): the ids
+        # that exist keep their pieces, text with other bytes cannot be encoded
+        pieces = pieces[: max(0, vocab_size - byte_base)]
         # id -> bytes
         self.id_to_bytes: List[Optional[bytes]] = [None] * vocab_size
         for i, p in enumerate(pieces):

@@ -326,6 +326,13 @@ _KAFILORN_F32 = ("norm1", "norm2", "hc1_in", "hc1_out", "hc1_mix", "hc2_in", "hc
 
 def _kafilorn_pack(cfg, get, device, dtype) -> Dict[str, torch.Tensor]:
     S = max(cfg.streams, 1)
+
+    def opt(name, n):   # a tensor the checkpoint may leave out: zeros (no correction, a sink of weight exp(0))
+        try:
+            return get(name)
+        except KeyError:
+            return torch.zeros(n)
+
     W: Dict[str, torch.Tensor] = {"embed": get("embed"), "lm_head": get("head"), "norm": get("final.norm").float(),
                                   "ones": torch.ones(S)}
     for i, L in enumerate(cfg.layers):
@@ -357,7 +364,7 @@ def _kafilorn_pack(cfg, get, device, dtype) -> Dict[str, torch.Tensor]:
         if f.kind == "dense":
             W[p + "w_up"], W[p + "w_down"] = get(c + "mlp.up"), get(c + "mlp.down")
         else:
-            W[p + "w_router"], W[p + "correction"] = get(c + "mlp.router"), get(c + "mlp.correction")
+            W[p + "w_router"], W[p + "correction"] = get(c + "mlp.router"), opt(c + "mlp.correction", f.experts)
             W[p + "w_gu"] = torch.stack([torch.cat([get(c + f"mlp.e{e}.gate"), get(c + f"mlp.e{e}.up")]) for e in range(f.experts)])
             W[p + "w_dn_e"] = torch.stack([get(c + f"mlp.e{e}.down") for e in range(f.experts)])
             if f.shared_ff:

@@ -29,10 +29,6 @@ def rms_div(x, eps):
     return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 def rotate(x, pos, base, dims):
     """Rotary position on the first `dims` entries of the last axis; entry i pairs with i + dims/2."""
     half = dims // 2
@@ -196,3 +192,100 @@ def forward(cfg, T, tokens, layer_out=None):
             layer_out(li, sum(xs))
     x = layer_norm(sum(xs), T["final.norm"], eps)
     return x @ f(T["head"]).T * cfg.get("logit_scale", 1.0)
+
+
+# ---------------------------------------------------------------------------------------------------
+# small random models for the tests (their own sizes; nothing here comes from the package)
+def mlstm_layer(heads=2, dim=8, vdim=8, gate_cap=15.0, mlp=None):
+    m = {"heads": heads, "dim": dim, "vdim": vdim}
+    if gate_cap:
+        m["gate_cap"] = gate_cap
+    return {"type": "mlstm", "mixer": m, "mlp": mlp}
+
+
+def attention_layer(heads=2, dim=8, rot_dim=4, vdim=8, q_rank=12, kv_rank=16, window=8, base=100.0, scale=None, kv_from=None,
+                    mlp=None):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "q_rank": q_rank, "kv_rank": kv_rank,
+         "scale": scale if scale is not None else (dim + rot_dim) ** -0.5}
+    if window:
+        m["mask"] = {"size": window}
+    if rot_dim:
+        m["rot"] = {"base": base, "dims": rot_dim}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return {"type": "latent_attention", "mixer": m, "mlp": mlp}
+
+
+def dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(experts=6, top=2, ff=16, groups=(3, 2), shared=16):
+    r = {"experts": experts, "top": top}
+    if groups:
+        r["groups"] = {"count": groups[0], "keep": groups[1]}
+    d = {"kind": "moe", "expert": {"ff": ff}, "router": r}
+    if shared:
+        d["shared"] = {"ff": shared}
+    return d
+
+
+def make_config(layers, width=32, vocab=96, streams=2, embed_scale=4.0, logit_scale=0.5, eps=1e-6):
+    c = {"architecture": "Kafilorn", "vocab": vocab, "width": width, "norm": {"eps": eps}, "embedding": {"scale": embed_scale},
+         "logit_scale": logit_scale, "layers": layers}
+    if streams:
+        c["streams"] = streams
+    return c
+
+
+def random_tensors(cfg, seed=0, dtype=torch.bfloat16):
+    """Random checkpoint tensors for `cfg` (bf16-representable values, as a checkpoint stores them)."""
+    g = torch.Generator().manual_seed(seed)
+    h, V, S = cfg["width"], cfg["vocab"], cfg.get("streams")
+
+    def mat(o, i, std=None):
+        return (torch.randn(o, i, generator=g) * (std if std is not None else i ** -0.5)).to(dtype)
+
+    def vec(n, lo=0.7, hi=1.3):
+        return (lo + (hi - lo) * torch.rand(n, generator=g)).to(dtype)
+
+    T = {"embed": mat(V, h, 1.0), "head": mat(V, h), "final.norm": vec(h)}
+    for i, L in enumerate(cfg["layers"]):
+        c, m, f = f"l{i}.", L["mixer"], L.get("mlp")
+        for q in ("1", "2") if f is not None else ("1",):
+            T[c + "norm" + q] = vec(h)
+            if S:
+                T[c + f"hc{q}.in"] = vec(S, 0.4 / S, 1.6 / S)
+                T[c + f"hc{q}.out"] = vec(S, 0.4, 1.1)
+                T[c + f"hc{q}.mix"] = (torch.eye(S) * 0.7 + torch.rand(S, S, generator=g) * (0.4 / S)).to(dtype)
+        if L["type"] == "mlstm":
+            H = m["heads"]
+            for k, n in (("q", m["dim"]), ("k", m["dim"]), ("v", m["vdim"]), ("g", m["vdim"])):
+                T[c + "mix." + k] = mat(H * n, h)
+            T[c + "mix.i"], T[c + "mix.f"] = mat(H, h, 2.0 * h ** -0.5), mat(H, h, 2.0 * h ** -0.5)
+            T[c + "mix.i.b"] = torch.randn(H, generator=g).to(dtype)
+            T[c + "mix.f.b"] = (2.0 + torch.randn(H, generator=g)).to(dtype)
+            T[c + "mix.norm"], T[c + "mix.o"] = vec(H * m["vdim"]), mat(h, H * m["vdim"])
+        else:
+            H = m["heads"]
+            T[c + "mix.dq"], T[c + "mix.dq.norm"] = mat(m["q_rank"], h), vec(m["q_rank"])
+            T[c + "mix.uq"] = mat(H * (m["dim"] + m["rot_dim"]), m["q_rank"], 2.0 * m["q_rank"] ** -0.5)
+            if m.get("kv_from") is None:
+                T[c + "mix.dkv"], T[c + "mix.dkv.norm"] = mat(m["kv_rank"] + m["rot_dim"], h), vec(m["kv_rank"])
+            T[c + "mix.uk"] = mat(H * m["dim"], m["kv_rank"], 2.0 * m["kv_rank"] ** -0.5)
+            T[c + "mix.uv"] = mat(H * m["vdim"], m["kv_rank"])
+            T[c + "mix.sink"] = torch.randn(H, generator=g).to(dtype)
+            T[c + "mix.o"] = mat(h, H * m["vdim"])
+        if f is None:
+            continue
+        if f["kind"] == "dense":
+            T[c + "mlp.up"], T[c + "mlp.down"] = mat(f["ff"], h), mat(h, f["ff"])
+        else:
+            E = f["router"]["experts"]
+            T[c + "mlp.router"] = mat(E, h, 3.0 * h ** -0.5)
+            T[c + "mlp.correction"] = (torch.randn(E, generator=g) * (0.6 / E)).to(dtype)
+            names = [f"mlp.e{e}." for e in range(E)] + (["mlp.shared."] if f.get("shared") else [])
+            for n in names:
+                ff = f["shared"]["ff"] if n == "mlp.shared." else f["expert"]["ff"]
+                T[c + n + "gate"], T[c + n + "up"], T[c + n + "down"] = mat(ff, h), mat(ff, h), mat(h, ff)
+    return T
