@@ -1,8 +1,10 @@
 """Engine-level prefill and decode throughput of two model families at equal layer sizes.
 
 `bench.py --arch-compare` runs this: for each size, a Vivepel configuration and the Llama configuration
-with the same width, heads, head size, feed-forward width, vocabulary and depth (random weights) go
-through the same engine path (`build_engine`, the scheduler, `ModelRunner.execute`, hipGraph decode):
+with the same width, heads, head size, feed-forward width, vocabulary and depth (random weights), and with
+`--arch-models ...,kafilorn` a Kafilorn of that width and depth (layers cycling mLSTM + dense, latent attention
++ experts, latent attention on the previous layer's cache + dense; latent ranks W/8 and 3W/8, 8 experts of
+width ff/4 with 2 chosen plus a shared one, two residual streams), go through the same engine path (`build_engine`, the scheduler, `ModelRunner.execute`, hipGraph decode):
 B prompts of P tokens are prefilled (in steps of the engine's token budget), then N tokens are
 decoded per sequence.  Reported per model: prefill tokens/s (prompt tokens / time in prefill steps)
 and decode tokens/s (B x decode steps / time in decode steps), from the runner's own step timers.
@@ -21,13 +23,18 @@ SIZES = {
 
 
 def _configs(size: str, chunk: int):
-    from .models.config import PRESETS, ModelConfig, vivepel_uniform
+    import dataclasses
+
+    from .models.config import PRESETS, ModelConfig, kafilorn_uniform, vivepel_uniform
 
     W, H, G, D, ff, V, L = SIZES[size]
     ll = ModelConfig(f"llama-{size}-{L}l", "llama", L, W, H, G, D, ff, V, 500000.0)
     vv = vivepel_uniform(f"vivepel-{size}-{L}l", L, W, H, G, D, ff, V, chunk=chunk)
-    PRESETS[ll.name], PRESETS[vv.name] = ll, vv
-    return ll, vv
+    kk = kafilorn_uniform(f"kafilorn-{size}-{L}l", (L + 2) // 3, W, H, V, ff, experts=8, top=2, expert_ff=ff // 4,
+                          window=chunk, streams=2, kv_rank=W // 8, q_rank=3 * W // 8, dim=D, rot_dim=D // 2)
+    kk = dataclasses.replace(kk, layers=kk.layers[:L])
+    PRESETS[ll.name], PRESETS[vv.name], PRESETS[kk.name] = ll, vv, kk
+    return ll, vv, kk
 
 
 def run_one(model: str, batch: int, prompt: int, new_tokens: int, warmup: int = 1, device: str = "cuda") -> dict:
@@ -73,8 +80,8 @@ def main(sizes=("2k", "8b"), batch: int = 32, prompt: int = 1024, new_tokens: in
          which=("llama", "vivepel")) -> dict:
     rows = []
     for size in sizes:
-        ll, vv = _configs(size, chunk)
-        for cfg in ([ll] if "llama" in which else []) + ([vv] if "vivepel" in which else []):
+        ll, vv, kk = _configs(size, chunk)
+        for cfg in [c for c, n in ((ll, "llama"), (vv, "vivepel"), (kk, "kafilorn")) if n in which]:
             r = run_one(cfg.name, batch, prompt, new_tokens)
             r["size"] = size
             rows.append(r)
@@ -82,5 +89,10 @@ def main(sizes=("2k", "8b"), batch: int = 32, prompt: int = 1024, new_tokens: in
     by = {(r["size"], r["model"].split("-")[0]): r for r in rows}
     ratio = {s: {k: round(by[(s, "vivepel")][k] / by[(s, "llama")][k], 3) for k in ("prefill_tok_s", "decode_tok_s")}
              for s in sizes if (s, "vivepel") in by and (s, "llama") in by}
-    return {"metric": "arch_compare", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
-            "chunk": chunk, "rows": rows, "vivepel_over_llama": ratio}
+    kratio = {s: {k: round(by[(s, "kafilorn")][k] / by[(s, "vivepel")][k], 3) for k in ("prefill_tok_s", "decode_tok_s")}
+              for s in sizes if (s, "kafilorn") in by and (s, "vivepel") in by}
+    out = {"metric": "arch_compare", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
+           "chunk": chunk, "rows": rows, "vivepel_over_llama": ratio}
+    if kratio:
+        out["kafilorn_over_vivepel"] = kratio
+    return out

@@ -14,8 +14,9 @@
 //   window_attention:  s_h(j) = (q_lat_h . c_j + q_rot_h . k_r,j) * scale for the keys j with
 //                  0 <= p - j < window (window 0: all j <= p); weights exp(s) / (sum exp(s) + exp(sink_h)),
 //                  the sink optional; out_h = sum_j w_h(j) c_j, written [H, T, R].
-//                  One workgroup per (token, group of heads); keys in tiles of 64 with an online softmax in
-//                  fp32.  A decode step is the same launch with one token per sequence.
+//                  Any dtype and shape: one workgroup per (token, group of heads), keys in tiles of 64 with an
+//                  online softmax in fp32 (mode 1, and what the matrix-core kernel below does not take).  A
+//                  decode step is the same launch with one token per sequence.
 #include "rows_f32.h"
 
 namespace {
@@ -229,6 +230,168 @@ __global__ __launch_bounds__(NT) void window_attention_kernel(AT* __restrict__ o
   }
 }
 
+
+// ---- bf16, matrix cores: the 16 rows of a tile are 16 heads of ONE token (every head reads the same cache
+// rows, so the heads are the M dimension of the products, for a decode row as for a prompt row).  A workgroup
+// of 4 waves takes (token, 16 heads); wave w visits the key tiles w, w + 4, ... (16 keys, one page: the tiles
+// are page-aligned) with its own online softmax:
+//   scores   S[16 heads x 16 keys] on MFMA 16x16x32 bf16: A = the staged query rows [latent | rotated part]
+//            from LDS, B = 16-byte loads straight from the token-major cache rows;
+//   weights  fp32; exp(S - running maximum), transposed through a per-wave LDS scratch into the A layout and
+//            split into two bf16 terms (hi + mid carries 16 mantissa bits), so the product with the values
+//            does not round the weights to bf16;
+//   values   the first R entries of the same cache rows, B fragments gathered from L1 (4 keys x 1 entry per
+//            lane), MFMA 16x16x16 bf16, fp32 accumulators [16 heads x R] in registers.
+// The four waves' partial results are merged in LDS (common maximum, summed denominators) and written once.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+constexpr int PST = 20;   // row stride of the weight scratch (floats): 16-byte aligned rows, no bank conflicts on the transpose
+
+template <int NB>
+__global__ __launch_bounds__(NT) void window_attention_tile_kernel(bf16_t* __restrict__ out,
+                                                                   const bf16_t* __restrict__ q_lat,
+                                                                   const float* __restrict__ q_rot,
+                                                                   const bf16_t* __restrict__ cache, WinArgs a) {
+  extern __shared__ float lds[];
+  const int R = a.R, Dr = a.Dr, E = R + Dr, H = a.H, T = a.T, BS = a.BS;
+  bf16_t* Qs = reinterpret_cast<bf16_t*>(lds);   // [16][E]
+  float* Pt = lds + 8 * E;                        // [NW][16][PST]
+  float* ML = Pt + NW * 16 * PST;                 // [NW][16][2] running (maximum, denominator) of each wave
+  float* INV = ML + NW * 16 * 2;                  // [16] 1 / total denominator
+  float* Acc = INV + 16;                          // [16][R]
+  const int t = blockIdx.x, h0 = blockIdx.y * 16;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int nh = min(16, H - h0);
+  if (a.slots[t] < 0) {
+    for (int i = tid; i < nh * R; i += NT) out[((size_t)(h0 + i / R) * T + t) * R + i % R] = 0;
+    return;
+  }
+  const int p = a.positions[t];
+  const int* bt = a.block_tables + (size_t)seq_of(a.q_starts, a.num_seqs, t) * a.max_blocks;
+  const int start = a.window > 0 ? max(0, p - a.window + 1) : 0;
+  const int jt0 = start & ~15;
+  for (int i = tid; i < 16 * E; i += NT) {
+    const int r = i / E, e = i % E, h = min(h0 + r, H - 1);
+    Qs[i] = e < R ? q_lat[((size_t)h * T + t) * R + e] : f2bf(q_rot[((size_t)t * H + h) * Dr + e - R]);
+  }
+  __syncthreads();
+  float m[4], l[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {   // the sink counts once: in wave 0
+    const bool sk = a.sink != nullptr && wave == 0;
+    m[r] = sk ? a.sink[min(h0 + 4 * grp + r, H - 1)] : -INFINITY;
+    l[r] = sk ? 1.f : 0.f;
+  }
+  f32x4 pacc[NB];
+#pragma unroll
+  for (int db = 0; db < NB; ++db) pacc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int nb = R >> 4, nks = E >> 5;
+  const int ntiles = ((p - jt0) >> 4) + 1;
+  float* pt = Pt + wave * 16 * PST;
+  const bf16_t* qrow = Qs + col * E + 8 * grp;
+  for (int ti = wave; ti < ntiles; ti += NW) {
+    const int jt = jt0 + 16 * ti;
+    const bf16_t* base = cache + ((size_t)bt[jt / BS] * BS + (jt % BS)) * E;   // rows jt .. jt + 15 of one page
+    const bf16_t* kp = base + (size_t)col * E + 8 * grp;
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    for (int ks = 0; ks < nks; ++ks)
+      s = mfma16x16x32(as_bf16x8(*reinterpret_cast<const uint4*>(qrow + 32 * ks)),
+                       as_bf16x8(*reinterpret_cast<const uint4*>(kp + 32 * ks)), s);
+    const int jj = jt + col;
+    const bool vis = jj >= start && jj <= p;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float x = vis ? s[r] * a.scale : -INFINITY;
+      const float mn = fmaxf(m[r], row16_max(x));
+      float pr = 0.f, c = 1.f;
+      if (mn != -INFINITY) {
+        pr = vis ? __expf(x - mn) : 0.f;
+        c = m[r] == -INFINITY ? 0.f : __expf(m[r] - mn);
+      }
+      l[r] = l[r] * c + row16_sum(pr);
+      m[r] = mn;
+      pt[(4 * grp + r) * PST + col] = pr;
+#pragma unroll
+      for (int db = 0; db < NB; ++db) pacc[db][r] *= c;
+    }
+    const f32x4 pa = *reinterpret_cast<const f32x4*>(pt + col * PST + 4 * grp);   // head `col`, keys 4 grp .. + 4
+    s16x4 ahi, amid;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bf16_t hi = f2bf(pa[i]);
+      ahi[i] = (short)hi;
+      amid[i] = (short)f2bf(pa[i] - bf2f(hi));
+    }
+    const bf16_t* vp = base + (size_t)(4 * grp) * E + col;
+#pragma unroll
+    for (int db = 0; db < NB; ++db) {
+      if (db < nb) {
+        const s16x4 b = {(short)vp[16 * db], (short)vp[E + 16 * db], (short)vp[2 * E + 16 * db], (short)vp[3 * E + 16 * db]};
+        pacc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ahi, b, pacc[db], 0, 0, 0);
+        pacc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(amid, b, pacc[db], 0, 0, 0);
+      }
+    }
+  }
+  // ---- merge the waves ----
+  if (col == 0) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      ML[(wave * 16 + 4 * grp + r) * 2] = m[r];
+      ML[(wave * 16 + 4 * grp + r) * 2 + 1] = l[r];
+    }
+  }
+  __syncthreads();
+  float f[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = 4 * grp + r;
+    float mg = -INFINITY;
+    for (int w = 0; w < NW; ++w) mg = fmaxf(mg, ML[(w * 16 + row) * 2]);
+    float lt = 0.f;
+    for (int w = 0; w < NW; ++w) {
+      const float mw = ML[(w * 16 + row) * 2];
+      if (mw != -INFINITY) lt += ML[(w * 16 + row) * 2 + 1] * __expf(mw - mg);
+    }
+    f[r] = m[r] == -INFINITY ? 0.f : __expf(m[r] - mg);
+    if (wave == 0 && col == 0) INV[row] = 1.0f / lt;
+  }
+  for (int w = 0; w < NW; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int db = 0; db < NB; ++db) {
+        if (db < nb) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int idx = (4 * grp + r) * R + 16 * db + col;
+            const float v = pacc[db][r] * f[r];
+            Acc[idx] = w == 0 ? v : Acc[idx] + v;
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  for (int i = tid; i < nh * R; i += NT) {
+    const int row = i / R;
+    out[((size_t)(h0 + row) * T + t) * R + i % R] = f2bf(Acc[i] * INV[row]);
+  }
+}
+
+template <int NB>
+int launch_tile(bf16_t* out, const bf16_t* q_lat, const float* q_rot, const bf16_t* cache, const WinArgs& a,
+                hipStream_t st) {
+  const int E = a.R + a.Dr;
+  const size_t lds = (size_t)(8 * E + NW * 16 * PST + NW * 16 * 2 + 16 + 16 * a.R) * sizeof(float);
+  if (lds > 48 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(window_attention_tile_kernel<NB>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+  }
+  dim3 grid(a.T, (a.H + 15) / 16);
+  window_attention_tile_kernel<NB><<<grid, NT, lds, st>>>(out, q_lat, q_rot, cache, a);
+  KA_CHECK_LAUNCH();
+}
+
 }  // namespace
 
 extern "C" int ka_latent_prep(void* cq, const void* proj, int T, int P, int Q, int R, int Dr, const float* w_q,
@@ -258,9 +421,20 @@ extern "C" int ka_rope_split_q(void* qn, float* qr, const void* q, const float* 
 extern "C" int ka_window_attention(void* out, const void* q_lat, const float* q_rot, const void* cache,
                                    const int* block_tables, const int* q_starts, int num_seqs, const int* positions,
                                    const int* slots, const float* sink, int T, int H, int R, int Dr, int BS,
-                                   int max_blocks, int window, float scale, int f32, hipStream_t st) {
+                                   int max_blocks, int window, float scale, int f32, int mode, hipStream_t st) {
   if (T <= 0) return 0;
   if (H <= 0 || R <= 0 || Dr < 0 || BS <= 0 || window < 0 || R > NT * MAX_ACC) return (int)hipErrorInvalidValue;
+  if (!f32 && mode == 0 && R % 16 == 0 && R <= 512 && (R + Dr) % 32 == 0 && BS % 16 == 0) {   // the matrix-core kernel
+    WinArgs a{block_tables, q_starts, num_seqs, positions, slots, sink, T, H, 16, R, Dr, BS, max_blocks, window, scale};
+    const int nb = R / 16;
+    bf16_t* o = (bf16_t*)out;
+    const bf16_t* ql = (const bf16_t*)q_lat;
+    const bf16_t* kc = (const bf16_t*)cache;
+    if (nb <= 4) return launch_tile<4>(o, ql, q_rot, kc, a, st);
+    if (nb <= 8) return launch_tile<8>(o, ql, q_rot, kc, a, st);
+    if (nb <= 16) return launch_tile<16>(o, ql, q_rot, kc, a, st);
+    return launch_tile<32>(o, ql, q_rot, kc, a, st);
+  }
   // heads per workgroup: as many as the accumulators (NT * MAX_ACC outputs), the 16 running values per wave
   // and 120 KB of LDS allow
   int HG = min(H, min(NT * MAX_ACC / R, 16 * NW));

@@ -125,7 +125,7 @@ _MIX_SIGS = {
     "ka_mlstm_scan": [P, P, I, I, I, I, P, P, P, P, P, P, I, P, I, I, I, F, I, P],
     "ka_latent_prep": [P, P, I, I, I, I, I, P, P, P, P, P, P, I, F, I, P],
     "ka_rope_split_q": [P, P, P, P, P, I, I, I, I, I, I, P],
-    "ka_window_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P],
+    "ka_window_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
     "ka_moe_route": [P, P, P, P, P, I, I, I, I, I, I, I, P],
     "ka_moe_rows": [P, P, P, P, P, P, P, I, I, I, I, I, P],
 }

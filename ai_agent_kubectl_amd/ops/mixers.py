@@ -168,6 +168,7 @@ def chunk_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 # ------------------------------------------------------------------------------------------------
 # residual streams, mLSTM, latent attention, grouped routing (csrc/streams_f32.hip, mlstm.hip,
 # attention_latent.hip, moe_route.hip)
+WINDOW_TILE = True   # bf16 window attention on the matrix cores where the shape allows (False: the per-token kernel)
 MOE_ROWS_MAX = 64    # token x expert rows served by the matrix-vector expert kernels (decode steps); more: sorted GEMMs
 
 
@@ -352,7 +353,8 @@ def window_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tens
     out = torch.empty((H, T, R), dtype=q_lat.dtype, device=q_lat.device)
     check(lib.ka_window_attention(_p(out), _p(q_lat), _p(q_rot), _p(cache), _p(block_tables), _p(q_starts),
                                   block_tables.shape[0], _p(positions), _p(slots), _p(sink), T, H, R, Dr, BS,
-                                  block_tables.shape[1], int(window), float(scale), _f32(q_lat), _stream()),
+                                  block_tables.shape[1], int(window), float(scale), _f32(q_lat),
+                                  0 if WINDOW_TILE else 1, _stream()),
           "window_attention")
     return out
 
@@ -387,7 +389,11 @@ def moe_experts(h: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, ids: 
     assert h.is_contiguous() and w_gu.is_contiguous() and w_down.is_contiguous() and w_gu.dtype == h.dtype == w_down.dtype
     assert w_down.shape == (E, W, ff) and ids.dtype == torch.int32 and w.dtype == torch.float32 and w.shape == ids.shape
     out = torch.zeros((T, W), dtype=torch.float32, device=h.device)
-    if T * top <= MOE_ROWS_MAX and W * 4 <= 60 * 1024 and top * ff * 4 <= 60 * 1024 and top <= 32:
+    rows_ok = W * 4 <= 60 * 1024 and top * ff * 4 <= 60 * 1024 and top <= 32
+    capturing = torch.cuda.is_current_stream_capturing()     # a graph cannot hold the sorted path's host read
+    if capturing and not rows_ok:
+        raise RuntimeError(f"moe_experts: width {W} / top {top} x ff {ff} outside the capturable kernels' limits")
+    if rows_ok and (capturing or T * top <= MOE_ROWS_MAX):
         lib = require_mixers()
         act = torch.empty((T * top, ff), dtype=h.dtype, device=h.device)
         check(lib.ka_moe_rows(_p(out), _p(act), _p(h), _p(w_gu), _p(w_down), _p(ids), _p(w), T, W, ff, top, _f32(h),

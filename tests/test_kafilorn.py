@@ -596,3 +596,55 @@ def test_graph_decode_matches_eager(tmp_path, dtype):
         if graphs:
             assert eng.runner.stats["graph_replays"] > 0
     assert got[0] == got[1]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,R,Dr,window,decode", [(16, 128, 32, 40, False), (4, 64, 0, 0, False), (20, 256, 64, 100, False),
+                                                  (40, 512, 64, 333, False), (16, 128, 32, 40, True), (33, 96, 32, 17, True),
+                                                  (8, 512, 64, 0, True)])
+def test_window_attention_matrix_core_kernel(H, R, Dr, window, decode):
+    """bf16 shapes the matrix-core kernel takes (heads below / at / above a 16-head tile and not multiples of it,
+    latents of 64 .. 512, windows that are not multiples of the 16-key tiles, none, shuffled pages), as prompt
+    portions of several sequences and as decode rows, against the torch reference on the same bf16 inputs."""
+    from ai_agent_kubectl_amd.ops import mixers, reference as ref
+
+    g = torch.Generator().manual_seed(H + R)
+    lens = [70, 5, 130] if not decode else [1, 1, 1, 1]
+    ctx = [200, 5, 300] if not decode else [97, 1, 260, 33]          # tokens in the cache after this step
+    bs, mb = 16, 20
+    nb = len(lens) * mb + 3
+    cache = (torch.randn(nb, bs, R + Dr, generator=g) * 0.7).to(torch.bfloat16)
+    bt = torch.randperm(nb, generator=g)[: len(lens) * mb].view(len(lens), mb).to(torch.int32)
+    pos, slots, starts = [], [], [0]
+    for i, (n, c) in enumerate(zip(lens, ctx)):
+        for p in range(c - n, c):
+            pos.append(p)
+            slots.append(int(bt[i, p // bs]) * bs + p % bs)
+        starts.append(starts[-1] + n)
+    T = len(pos) + 3                                                  # three padding rows
+    pos_t = torch.tensor(pos + [0] * 3, dtype=torch.int32)
+    slots_t = torch.tensor(slots + [-1] * 3, dtype=torch.int32)
+    q_lat = (torch.randn(H, T, R, generator=g) * 0.5).to(torch.bfloat16)
+    q_rot = torch.randn(T, H, Dr, generator=g)
+    sink = torch.randn(H, generator=g)
+    q_starts = None if decode else torch.tensor(starts, dtype=torch.int32)
+    if decode:
+        T = len(lens)
+        q_lat, q_rot, pos_t, slots_t = q_lat[:, :T].contiguous(), q_rot[:T].contiguous(), pos_t[:T], slots_t[:T]
+    scale = (R + Dr) ** -0.5 * 2
+    want = ref.window_attention(q_lat.float(), q_rot.to(torch.bfloat16).float(), cache.float(), bt, q_starts, pos_t, slots_t,
+                                sink, window, scale)
+    dev = lambda x: None if x is None else x.cuda()   # noqa: E731
+    outs = {}
+    for tile in (True, False):
+        mixers.WINDOW_TILE = tile
+        try:
+            outs[tile] = mixers.window_attention(dev(q_lat), dev(q_rot), dev(cache), dev(bt), dev(q_starts), dev(pos_t),
+                                                 dev(slots_t), dev(sink), window, scale).float().cpu()
+        finally:
+            mixers.WINDOW_TILE = True
+    n_real = len(pos) if not decode else T
+    for tile, got in outs.items():
+        err = (got[:, :n_real] - want[:, :n_real]).abs().max() / want.abs().max()
+        assert err < (1.5e-2 if tile else 1e-2), (tile, float(err))
+        assert torch.all(got[:, n_real:] == 0)
