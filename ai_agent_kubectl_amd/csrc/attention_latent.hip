@@ -240,10 +240,13 @@ __global__ __launch_bounds__(NT) void window_attention_kernel(AT* __restrict__ o
 //   weights  fp32; exp(S - running maximum), transposed through a per-wave LDS scratch into the A layout and
 //            split into two bf16 terms (hi + mid carries 16 mantissa bits), so the product with the values
 //            does not round the weights to bf16;
-//   values   the first R entries of the same cache rows, B fragments gathered from L1 (4 keys x 1 entry per
-//            lane), MFMA 16x16x16 bf16, fp32 accumulators [16 heads x R] in registers.
+//   values   the first R entries of the same cache rows: the key fragments already in registers are written to
+//            a per-wave LDS tile entry-major, B fragments are 8-byte LDS reads; MFMA 16x16x16 bf16, fp32
+//            accumulators [16 heads x R] in registers.
 // The four waves' partial results are merged in LDS (common maximum, summed denominators) and written once.
 typedef short s16x4 __attribute__((ext_vector_type(4)));
+constexpr int KU = 6;    // key fragments requested together
+constexpr int VST = 20;  // keys per value entry in a wave's staged tile (16 + padding: 8-byte aligned rows)
 constexpr int PST = 20;   // row stride of the weight scratch (floats): 16-byte aligned rows, no bank conflicts on the transpose
 
 template <int NB>
@@ -253,11 +256,13 @@ __global__ __launch_bounds__(NT) void window_attention_tile_kernel(bf16_t* __res
                                                                    const bf16_t* __restrict__ cache, WinArgs a) {
   extern __shared__ float lds[];
   const int R = a.R, Dr = a.Dr, E = R + Dr, H = a.H, T = a.T, BS = a.BS;
-  bf16_t* Qs = reinterpret_cast<bf16_t*>(lds);   // [16][E]
-  float* Pt = lds + 8 * E;                        // [NW][16][PST]
+  const int QST = E + 8;                          // query row stride: 16 more bytes, so the 16 rows' fragments fall in different banks
+  bf16_t* Qs = reinterpret_cast<bf16_t*>(lds);   // [16][QST]
+  float* Pt = lds + 8 * QST;                      // [NW][16][PST]
   float* ML = Pt + NW * 16 * PST;                 // [NW][16][2] running (maximum, denominator) of each wave
   float* INV = ML + NW * 16 * 2;                  // [16] 1 / total denominator
-  float* Acc = INV + 16;                          // [16][R]
+  float* Acc = INV + 16;                          // [16][R] the merged result; the same memory holds, during the key
+  bf16_t* vs = reinterpret_cast<bf16_t*>(Acc) + (size_t)(threadIdx.x >> 6) * R * VST;   // loop, each wave's value tile [R][VST]
   const int t = blockIdx.x, h0 = blockIdx.y * 16;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, grp = lane >> 4;
@@ -272,7 +277,7 @@ __global__ __launch_bounds__(NT) void window_attention_tile_kernel(bf16_t* __res
   const int jt0 = start & ~15;
   for (int i = tid; i < 16 * E; i += NT) {
     const int r = i / E, e = i % E, h = min(h0 + r, H - 1);
-    Qs[i] = e < R ? q_lat[((size_t)h * T + t) * R + e] : f2bf(q_rot[((size_t)t * H + h) * Dr + e - R]);
+    Qs[r * QST + e] = e < R ? q_lat[((size_t)h * T + t) * R + e] : f2bf(q_rot[((size_t)t * H + h) * Dr + e - R]);
   }
   __syncthreads();
   float m[4], l[4];
@@ -288,17 +293,40 @@ __global__ __launch_bounds__(NT) void window_attention_tile_kernel(bf16_t* __res
   const int nb = R >> 4, nks = E >> 5;
   const int ntiles = ((p - jt0) >> 4) + 1;
   float* pt = Pt + wave * 16 * PST;
-  const bf16_t* qrow = Qs + col * E + 8 * grp;
+  const bf16_t* qrow = Qs + col * QST + 8 * grp;
   for (int ti = wave; ti < ntiles; ti += NW) {
     const int jt = jt0 + 16 * ti;
     const bf16_t* base = cache + ((size_t)bt[jt / BS] * BS + (jt % BS)) * E;   // rows jt .. jt + 15 of one page
     const bf16_t* kp = base + (size_t)col * E + 8 * grp;
+    // the key fragments are requested KU at a time; the first R entries of a key row are also its value, so each
+    // fragment of the latent part is written to the wave's LDS tile transposed (entry-major, 16 keys side by
+    // side): the B operand of weights x values is then one 8-byte LDS read
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
-    for (int ks = 0; ks < nks; ++ks)
-      s = mfma16x16x32(as_bf16x8(*reinterpret_cast<const uint4*>(qrow + 32 * ks)),
-                       as_bf16x8(*reinterpret_cast<const uint4*>(kp + 32 * ks)), s);
+    for (int c0 = 0; c0 < nks; c0 += KU) {
+      uint4 kf[KU];
+#pragma unroll
+      for (int u = 0; u < KU; ++u) kf[u] = *reinterpret_cast<const uint4*>(kp + 32 * min(c0 + u, nks - 1));
+#pragma unroll
+      for (int u = 0; u < KU; ++u) {
+        const int ks = c0 + u;
+        if (ks < nks) {
+          s = mfma16x16x32(as_bf16x8(*reinterpret_cast<const uint4*>(qrow + 32 * ks)), as_bf16x8(kf[u]), s);
+          const int d0 = 32 * ks + 8 * grp;
+          if (d0 < R) {
+            bf16_t* dst = vs + (size_t)d0 * VST + col;
+            const uint32_t wd[4] = {kf[u].x, kf[u].y, kf[u].z, kf[u].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              dst[(2 * i) * VST] = (bf16_t)(wd[i] & 0xffffu);
+              dst[(2 * i + 1) * VST] = (bf16_t)(wd[i] >> 16);
+            }
+          }
+        }
+      }
+    }
     const int jj = jt + col;
     const bool vis = jj >= start && jj <= p;
+    float cr[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const float x = vis ? s[r] * a.scale : -INFINITY;
@@ -311,8 +339,13 @@ __global__ __launch_bounds__(NT) void window_attention_tile_kernel(bf16_t* __res
       l[r] = l[r] * c + row16_sum(pr);
       m[r] = mn;
       pt[(4 * grp + r) * PST + col] = pr;
+      cr[r] = c;
+    }
+    if (__any(cr[0] != 1.f || cr[1] != 1.f || cr[2] != 1.f || cr[3] != 1.f)) {   // a maximum moved (rare after the first tiles)
 #pragma unroll
-      for (int db = 0; db < NB; ++db) pacc[db][r] *= c;
+      for (int db = 0; db < NB; ++db)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) pacc[db][r] *= cr[r];
     }
     const f32x4 pa = *reinterpret_cast<const f32x4*>(pt + col * PST + 4 * grp);   // head `col`, keys 4 grp .. + 4
     s16x4 ahi, amid;
@@ -322,17 +355,18 @@ __global__ __launch_bounds__(NT) void window_attention_tile_kernel(bf16_t* __res
       ahi[i] = (short)hi;
       amid[i] = (short)f2bf(pa[i] - bf2f(hi));
     }
-    const bf16_t* vp = base + (size_t)(4 * grp) * E + col;
+    const bf16_t* vrd = vs + (size_t)col * VST + 4 * grp;   // entry 16 db + col, keys 4 grp .. + 4
 #pragma unroll
     for (int db = 0; db < NB; ++db) {
       if (db < nb) {
-        const s16x4 b = {(short)vp[16 * db], (short)vp[E + 16 * db], (short)vp[2 * E + 16 * db], (short)vp[3 * E + 16 * db]};
+        const s16x4 b = *reinterpret_cast<const s16x4*>(vrd + (size_t)16 * db * VST);
         pacc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ahi, b, pacc[db], 0, 0, 0);
         pacc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(amid, b, pacc[db], 0, 0, 0);
       }
     }
   }
   // ---- merge the waves ----
+  __syncthreads();   // every wave is done with its value tile: the memory becomes the merged result
   if (col == 0) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -381,7 +415,9 @@ template <int NB>
 int launch_tile(bf16_t* out, const bf16_t* q_lat, const float* q_rot, const bf16_t* cache, const WinArgs& a,
                 hipStream_t st) {
   const int E = a.R + a.Dr;
-  const size_t lds = (size_t)(8 * E + NW * 16 * PST + NW * 16 * 2 + 16 + 16 * a.R) * sizeof(float);
+  // the value tiles (NW x R x VST bf16) and the merged result (16 x R fp32) share memory
+  const size_t tail = (size_t)a.R * (NW * VST * 2 > 16 * 4 ? NW * VST * 2 : 16 * 4);
+  const size_t lds = (size_t)(8 * (E + 8) + NW * 16 * PST + NW * 16 * 2 + 16) * sizeof(float) + tail;
   if (lds > 48 * 1024) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(window_attention_tile_kernel<NB>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

@@ -11,7 +11,8 @@
 //   moe_gate_up / moe_down:  for step sizes of a few rows (decode), the chosen experts as matrix-vector
 //               products straight from the stacked expert weights, no routing lists and no host read, so a
 //               decode step can be captured: act[t, k] = silu(gate_e h) * (up_e h) with e = ids[t, k], then
-//               out[t] = sum_k w[t, k] down_e act[t, k] in fp32.
+//               out[t] = sum_k w[t, k] down_e act[t, k] in fp32.  Any dtype; the fp32 engine's path.
+//   moe_grouped:  the same step in bf16 on the matrix cores, rows grouped by expert (below).
 #include "rows_f32.h"
 
 namespace {
@@ -154,6 +155,72 @@ __global__ __launch_bounds__(NT) void moe_down_kernel(float* __restrict__ out, c
   }
 }
 
+
+// ---- bf16, matrix cores: the experts of a decode-sized step, grouped by expert so that every expert's weights
+// are read once.  A workgroup takes (expert e, 64 output features): it lists the (token, choice) rows routed to e
+// and runs them, 16 at a time, as the M rows of MFMA 16x16x32 products against the expert's weight rows (B
+// fragments are 16-byte loads straight from the stacked weights, A fragments 16-byte loads of the gathered rows).
+//   MODE 0: act[row] = silu(gate_e x) * (up_e x), x = h[row / top]         (bf16 out, K = width, N = ff)
+//   MODE 1: yk[row]  = down_e act[row]                                      (fp32 out, K = ff,    N = width)
+// and `moe_combine` sums a token's rows in the order of its choices with the router weights.  No host read and no
+// data-dependent launch shape: a decode step with experts can be captured into a graph.
+constexpr int GROUP_MAX_ROWS = 1024;
+
+template <int MODE>
+__global__ __launch_bounds__(NT) void moe_group_kernel(void* __restrict__ out, const bf16_t* __restrict__ x,
+                                                       const bf16_t* __restrict__ w, const int* __restrict__ ids,
+                                                       int rows_, int K, int N, int top) {
+  __shared__ int list[GROUP_MAX_ROWS];
+  __shared__ int cnt;
+  const int e = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  if (tid == 0) cnt = 0;
+  __syncthreads();
+  for (int r = tid; r < rows_; r += NT)
+    if (ids[r] == e) list[atomicAdd(&cnt, 1)] = r;
+  __syncthreads();
+  const int n = cnt;
+  if (n == 0) return;
+  const int n0 = blockIdx.y * 64 + wave * 16;
+  if (n0 >= N) return;
+  const int nc = min(n0 + col, N - 1);
+  const bf16_t* wg = w + ((size_t)e * (MODE == 0 ? 2 * N : N) + nc) * K + 8 * grp;
+  const bf16_t* wu = wg + (size_t)N * K;   // MODE 0: the up rows follow the gate rows
+  for (int mt = 0; mt * 16 < n; ++mt) {
+    const int ridx = list[min(mt * 16 + col, n - 1)];
+    const bf16_t* xr = x + (size_t)(MODE == 0 ? ridx / top : ridx) * K + 8 * grp;
+    f32x4 ag = {0.f, 0.f, 0.f, 0.f}, au = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+    for (int k0 = 0; k0 < K; k0 += 32) {
+      const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(xr + k0));
+      ag = mfma16x16x32(a, as_bf16x8(*reinterpret_cast<const uint4*>(wg + k0)), ag);
+      if constexpr (MODE == 0) au = mfma16x16x32(a, as_bf16x8(*reinterpret_cast<const uint4*>(wu + k0)), au);
+    }
+    if (n0 + col < N) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = mt * 16 + 4 * grp + r;
+        if (row < n) {
+          const size_t at = (size_t)list[row] * N + n0 + col;
+          if constexpr (MODE == 0) reinterpret_cast<bf16_t*>(out)[at] = f2bf(ag[r] / (1.f + expf(-ag[r])) * au[r]);
+          else reinterpret_cast<float*>(out)[at] = ag[r];
+        }
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(NT) void moe_combine_kernel(float* __restrict__ out, const float* __restrict__ yk,
+                                                         const float* __restrict__ wts, int width, int top) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < width; c += NT) {
+    float s = 0.f;
+    for (int k = 0; k < top; ++k) s += wts[(size_t)t * top + k] * yk[((size_t)t * top + k) * width + c];
+    out[(size_t)t * width + c] = s;
+  }
+}
+
 }  // namespace
 
 extern "C" int ka_moe_route(int* ids, float* wts, const void* h, const float* wr, const float* correction, int T,
@@ -181,5 +248,16 @@ extern "C" int ka_moe_rows(float* out, void* act, const void* h, const void* w_g
     moe_gate_up_kernel<bf16_t><<<g1, NT, l1, st>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, ids, width, ff, top);
     moe_down_kernel<bf16_t><<<g2, NT, l2, st>>>(out, (const bf16_t*)act, (const bf16_t*)w_down, ids, wts, width, ff, top);
   }
+  KA_CHECK_LAUNCH();
+}
+
+// bf16 only; `act` [T * top, ff] bf16 and `yk` [T * top, width] fp32 are scratch
+extern "C" int ka_moe_grouped(float* out, void* act, float* yk, const void* h, const void* w_gu, const void* w_down,
+                              const int* ids, const float* wts, int T, int width, int ff, int top, int E, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (T * top > GROUP_MAX_ROWS || width % 32 || ff % 32 || top <= 0 || E <= 0) return (int)hipErrorInvalidValue;
+  moe_group_kernel<0><<<dim3(E, (ff + 63) / 64), NT, 0, st>>>(act, (const bf16_t*)h, (const bf16_t*)w_gu, ids, T * top, width, ff, top);
+  moe_group_kernel<1><<<dim3(E, (width + 63) / 64), NT, 0, st>>>(yk, (const bf16_t*)act, (const bf16_t*)w_down, ids, T * top, ff, width, top);
+  moe_combine_kernel<<<T, NT, 0, st>>>(out, yk, wts, width, top);
   KA_CHECK_LAUNCH();
 }

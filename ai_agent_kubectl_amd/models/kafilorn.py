@@ -105,7 +105,7 @@ class KafilornModel:
             raise RuntimeError("mLSTM layer without state slots: the runner must call alloc_state and pass state_slots")
         HD, HV = m.heads * m.dim, m.heads * m.vdim
         proj = F.linear(h, L["w_proj"])                                # [T, q | k | v | g]
-        gates = mixers.mlstm_gates(h, L["w_if"], L["b_if"], m.gate_cap)
+        gates = mixers.mlstm_gates(h, L["w_if"], L["b_if"], m.gate_cap, L.get("w_if_lp"))
         S, n, mx = self.state[li]
         o = mixers.mlstm_scan(proj, 0, HD, 2 * HD, gates, S, n, mx, meta.state_slots,
                               None if meta.is_decode else meta.q_starts, meta.positions, m.heads, m.dim, m.vdim,

@@ -312,7 +312,7 @@ def load_vivepel_safetensors(path: str, cfg, device="cpu", dtype=torch.bfloat16)
 # Kafilorn.  Engine layout per layer `layers.<i>.` (activation dtype unless marked fp32):
 #   norm1, norm2, hc{1,2}_in [S], hc{1,2}_out [S], hc{1,2}_mix [S, S]                         fp32
 #   mLSTM:  w_proj [q; k; v; g rows, W] (one GEMM), w_if [2H, W] + b_if [2H] fp32 (input gates, then forget
-#           gates), hnorm [H * Dv] fp32, wo [W, H * Dv]
+#           gates; w_if_lp: the checkpoint's bf16 values of w_if, bf16 engine only), hnorm [H * Dv] fp32, wo [W, H * Dv]
 #   latent attention:  w_dn [dq rows; dkv rows, W] (one GEMM; dq alone when the layer borrows another layer's
 #           cache), q_norm [Q] / kv_norm [R] / sink [H] / inv_freq fp32, w_uq [H * (D + Dr), Q],
 #           w_uk [H, D, R], w_uv [H, Dv, R], wo [W, H * Dv]
@@ -345,6 +345,8 @@ def _kafilorn_pack(cfg, get, device, dtype) -> Dict[str, torch.Tensor]:
             W[p + "w_proj"] = torch.cat([get(c + "mix.q"), get(c + "mix.k"), get(c + "mix.v"), get(c + "mix.g")])
             W[p + "w_if"] = torch.cat([get(c + "mix.i"), get(c + "mix.f")])
             W[p + "b_if"] = torch.cat([get(c + "mix.i.b"), get(c + "mix.f.b")])
+            if dtype == torch.bfloat16 and W[p + "w_if"].dtype == torch.bfloat16:
+                W[p + "w_if_lp"] = W[p + "w_if"]    # the stored bf16 values, for the matrix cores (w_if becomes fp32 below)
             W[p + "hnorm"], W[p + "wo"] = get(c + "mix.norm"), get(c + "mix.o")
         else:
             own = m.kv_from < 0

@@ -122,12 +122,14 @@ _MIX_SIGS = {
     "ka_silu_mul_rows": [P, P, I, I, I, P],
     "ka_headnorm_gate": [P, P, P, I, I, P, I, I, I, F, I, P],
     "ka_mlstm_gates": [P, P, P, P, I, I, I, F, I, P],
-    "ka_mlstm_scan": [P, P, I, I, I, I, P, P, P, P, P, P, I, P, I, I, I, F, I, P],
+    "ka_mlstm_gates_mfma": [P, P, P, P, I, I, I, F, P],
+    "ka_mlstm_scan": [P, P, I, I, I, I, P, P, P, P, P, P, P, I, P, I, I, I, F, I, P],
     "ka_latent_prep": [P, P, I, I, I, I, I, P, P, P, P, P, P, I, F, I, P],
     "ka_rope_split_q": [P, P, P, P, P, I, I, I, I, I, I, P],
     "ka_window_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
     "ka_moe_route": [P, P, P, P, P, I, I, I, I, I, I, I, P],
     "ka_moe_rows": [P, P, P, P, P, P, P, I, I, I, I, I, P],
+    "ka_moe_grouped": [P, P, P, P, P, P, P, P, I, I, I, I, I, P],
 }
 MIXERS_LIB = os.path.join(LIB_DIR, "libkagent_mixers.so")
 _mix: Optional[ctypes.CDLL] = None

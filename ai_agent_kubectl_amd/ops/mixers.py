@@ -169,6 +169,7 @@ def chunk_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 # residual streams, mLSTM, latent attention, grouped routing (csrc/streams_f32.hip, mlstm.hip,
 # attention_latent.hip, moe_route.hip)
 WINDOW_TILE = True   # bf16 window attention on the matrix cores where the shape allows (False: the per-token kernel)
+MOE_GROUP_MAX = 1024  # bf16: token x expert rows served by the expert-grouped matrix-core kernels (decode steps)
 MOE_ROWS_MAX = 64    # token x expert rows served by the matrix-vector expert kernels (decode steps); more: sorted GEMMs
 
 
@@ -240,12 +241,22 @@ def silu_mul(gu: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def mlstm_gates(h: torch.Tensor, w_if: torch.Tensor, b_if: torch.Tensor, cap: float) -> torch.Tensor:
-    """[T, 2H] fp32: log input gates (soft-capped), then log forget gates logsigmoid(soft-capped)."""
+def mlstm_gates(h: torch.Tensor, w_if: torch.Tensor, b_if: torch.Tensor, cap: float,
+                w_lp: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[T, 2H] fp32: log input gates (soft-capped), then log forget gates logsigmoid(soft-capped).  w_lp: a bf16
+    copy of w_if holding the same values (weights that a checkpoint stores in bf16): bf16 rows then run on the
+    matrix cores, where products of bf16 inputs are exact and accumulate in fp32."""
     if _ref(h):
         return ref.mlstm_gates(h, w_if, b_if, cap)
     lib = require_mixers()
     T, W = h.shape
+    if (w_lp is not None and h.dtype == torch.bfloat16 and w_lp.dtype == torch.bfloat16 and W % 128 == 0
+            and w_lp.shape[0] <= 128):
+        assert h.is_contiguous() and w_lp.is_contiguous() and w_lp.shape == w_if.shape and b_if.dtype == torch.float32
+        out = torch.empty((T, w_lp.shape[0]), dtype=torch.float32, device=h.device)
+        check(lib.ka_mlstm_gates_mfma(_p(out), _p(h), _p(w_lp), _p(b_if), T, W, w_lp.shape[0] // 2, float(cap), _stream()),
+              "mlstm_gates_mfma")
+        return out
     assert h.is_contiguous() and w_if.dtype == torch.float32 and w_if.shape[1] == W and w_if.is_contiguous()
     assert b_if.dtype == torch.float32 and b_if.numel() == w_if.shape[0] and w_if.shape[0] % 2 == 0
     out = torch.empty((T, w_if.shape[0]), dtype=torch.float32, device=h.device)
@@ -275,7 +286,8 @@ def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gates: to
     assert (q_starts is None and nseq <= T) or (q_starts is not None and q_starts.dtype == torch.int32
                                                  and q_starts.shape[0] == nseq + 1)
     out = torch.zeros((T, H * Dv), dtype=torch.float32, device=proj.device)
-    check(lib.ka_mlstm_scan(_p(out), _p(proj), P, q_off, k_off, v_off, _p(gates), _p(st_S), _p(st_n), _p(st_m),
+    dec = torch.empty((T, H, 3), dtype=torch.float32, device=proj.device)   # per row: forget factor, input factor, exp(-max)
+    check(lib.ka_mlstm_scan(_p(out), _p(proj), P, q_off, k_off, v_off, _p(gates), _p(dec), _p(st_S), _p(st_n), _p(st_m),
                             _p(seq_slots), _p(q_starts), nseq, _p(positions), H, D, Dv, float(qscale), _f32(proj),
                             _stream()), "mlstm_scan")
     return out
@@ -378,8 +390,8 @@ def moe_route(h: torch.Tensor, w_router: torch.Tensor, correction: Optional[torc
 
 def moe_experts(h: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """sum_k w[t, k] * expert_{ids[t, k]}(h[t]) -> [T, W] fp32; w_gu [E, 2 ff, W] (gate rows, then up rows),
-    w_down [E, W, ff].  A few rows (decode): matrix-vector kernels straight from the stacked weights, no host
-    read, capturable.  More: rows sorted by expert, one read of the per-expert counts, one vendor GEMM pair per
+    w_down [E, W, ff].  Decode-sized steps: in bf16 the rows grouped by expert on the matrix cores, otherwise
+    matrix-vector kernels straight from the stacked weights; neither reads the host, both are capturable.  More: rows sorted by expert, one read of the per-expert counts, one vendor GEMM pair per
     expert segment, weighted scatter-add in fp32."""
     if _ref(h):
         return ref.moe_experts(h, w_gu, w_down, ids, w)
@@ -389,6 +401,13 @@ def moe_experts(h: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, ids: 
     assert h.is_contiguous() and w_gu.is_contiguous() and w_down.is_contiguous() and w_gu.dtype == h.dtype == w_down.dtype
     assert w_down.shape == (E, W, ff) and ids.dtype == torch.int32 and w.dtype == torch.float32 and w.shape == ids.shape
     out = torch.zeros((T, W), dtype=torch.float32, device=h.device)
+    if h.dtype == torch.bfloat16 and T * top <= MOE_GROUP_MAX and W % 32 == 0 and ff % 32 == 0:
+        lib = require_mixers()   # rows grouped by expert on the matrix cores: every expert's weights read once
+        act = torch.empty((T * top, ff), dtype=h.dtype, device=h.device)
+        yk = torch.empty((T * top, W), dtype=torch.float32, device=h.device)
+        check(lib.ka_moe_grouped(_p(out), _p(act), _p(yk), _p(h), _p(w_gu), _p(w_down), _p(ids), _p(w), T, W, ff, top, E,
+                                 _stream()), "moe_grouped")
+        return out
     rows_ok = W * 4 <= 60 * 1024 and top * ff * 4 <= 60 * 1024 and top <= 32
     capturing = torch.cuda.is_current_stream_capturing()     # a graph cannot hold the sorted path's host read
     if capturing and not rows_ok:

@@ -648,3 +648,37 @@ def test_window_attention_matrix_core_kernel(H, R, Dr, window, decode):
         err = (got[:, :n_real] - want[:, :n_real]).abs().max() / want.abs().max()
         assert err < (1.5e-2 if tile else 1e-2), (tile, float(err))
         assert torch.all(got[:, n_real:] == 0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T_rows,top", [(3, 2), (40, 3), (300, 2)])
+def test_experts_grouped_on_matrix_cores(T_rows, top):
+    """bf16 decode-sized steps: rows grouped by expert (fewer / more than a 16-row tile per expert, an expert with
+    no row at all) against the fp32 sum over the same bf16 weights."""
+    from ai_agent_kubectl_amd.ops import mixers, reference as ref
+
+    g = torch.Generator().manual_seed(T_rows)
+    E, W, ff = 6, 64, 96
+    h = torch.randn(T_rows, W, generator=g).to(torch.bfloat16)
+    w_gu = (torch.randn(E, 2 * ff, W, generator=g) * 0.3).to(torch.bfloat16)
+    w_dn = (torch.randn(E, W, ff, generator=g) * 0.3).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(E - 1, generator=g)[:top] for _ in range(T_rows)]).to(torch.int32)   # expert 5 idle
+    w = torch.rand(T_rows, top, generator=g)
+    want = ref.moe_experts(h.float(), w_gu.float(), w_dn.float(), ids, w)
+    got = mixers.moe_experts(h.cuda(), w_gu.cuda(), w_dn.cuda(), ids.cuda(), w.cuda()).cpu()
+    assert (got - want).abs().max() < 2e-2 * want.abs().max()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T_rows,W,H", [(5, 128, 2), (100, 256, 12), (33, 384, 40)])
+def test_gates_on_matrix_cores(T_rows, W, H):
+    from ai_agent_kubectl_amd.ops import mixers, reference as ref
+
+    g = torch.Generator().manual_seed(W)
+    h = torch.randn(T_rows, W, generator=g).to(torch.bfloat16)
+    w = (torch.randn(2 * H, W, generator=g) * 0.2).to(torch.bfloat16)
+    b = torch.randn(2 * H, generator=g)
+    want = ref.mlstm_gates(h.float(), w.float(), b, 6.0)
+    slow = mixers.mlstm_gates(h.cuda(), w.float().cuda(), b.cuda(), 6.0).cpu()
+    fast = mixers.mlstm_gates(h.cuda(), w.float().cuda(), b.cuda(), 6.0, w.cuda()).cpu()
+    assert torch.allclose(slow, want, rtol=1e-4, atol=1e-4) and torch.allclose(fast, want, rtol=1e-4, atol=1e-4)
