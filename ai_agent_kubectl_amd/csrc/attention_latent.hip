@@ -275,9 +275,16 @@ __global__ __launch_bounds__(NT) void window_attention_tile_kernel(bf16_t* __res
   const int* bt = a.block_tables + (size_t)seq_of(a.q_starts, a.num_seqs, t) * a.max_blocks;
   const int start = a.window > 0 ? max(0, p - a.window + 1) : 0;
   const int jt0 = start & ~15;
-  for (int i = tid; i < 16 * E; i += NT) {
-    const int r = i / E, e = i % E, h = min(h0 + r, H - 1);
-    Qs[r * QST + e] = e < R ? q_lat[((size_t)h * T + t) * R + e] : f2bf(q_rot[((size_t)t * H + h) * Dr + e - R]);
+  {   // the 16 query rows: the latent parts in 16-byte pieces, the rotated parts converted to bf16
+    const int c8 = R >> 3;
+    for (int i = tid; i < 16 * c8; i += NT) {
+      const int r = i / c8, c = i - r * c8, h = min(h0 + r, H - 1);
+      *reinterpret_cast<uint4*>(Qs + r * QST + 8 * c) = *reinterpret_cast<const uint4*>(q_lat + ((size_t)h * T + t) * R + 8 * c);
+    }
+    for (int i = tid; i < 16 * Dr; i += NT) {
+      const int r = i / Dr, e = i - r * Dr, h = min(h0 + r, H - 1);
+      Qs[r * QST + R + e] = f2bf(q_rot[((size_t)t * H + h) * Dr + e]);
+    }
   }
   __syncthreads();
   float m[4], l[4];
@@ -405,9 +412,15 @@ __global__ __launch_bounds__(NT) void window_attention_tile_kernel(bf16_t* __res
     }
     __syncthreads();
   }
-  for (int i = tid; i < nh * R; i += NT) {
-    const int row = i / R;
-    out[((size_t)(h0 + row) * T + t) * R + i % R] = f2bf(Acc[i] * INV[row]);
+  {
+    const int c4 = R >> 2;   // four results per thread and store
+    for (int i = tid; i < nh * c4; i += NT) {
+      const int row = i / c4, c = i - row * c4;
+      const f32x4 v = *reinterpret_cast<const f32x4*>(Acc + row * R + 4 * c);
+      const float inv = INV[row];
+      uint2 pk = {pack2(v[0] * inv, v[1] * inv), pack2(v[2] * inv, v[3] * inv)};
+      *reinterpret_cast<uint2*>(out + ((size_t)(h0 + row) * T + t) * R + 4 * c) = pk;
+    }
   }
 }
 

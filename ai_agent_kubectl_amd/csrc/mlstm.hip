@@ -12,9 +12,8 @@
 // one wave per output), soft-capped by cap * tanh(. / cap) when cap > 0; the forget gate then through
 // log-sigmoid.  `mlstm_scan`: the recurrence over the rows that each sequence brings to this step, from the
 // state in the sequence's slot and back into it; a row at position 0 starts from the zero state, so a slot
-// needs no clearing between requests.  The scalar chain (running maximum, the two factors of every row) runs
-// once per (sequence, head) in a launch of its own; then one workgroup per (sequence, head, 16 value columns):
-// a column is held by 16 lanes, each with D / 16 rows of S in registers; rows are staged 16 .. 64 at a time in LDS.
+// needs no clearing between requests.  The scalar chain (running maximum, the rows' factors) runs once per
+// (sequence, head) in a launch of its own, as a parallel scan; the state update follows (below).
 // The same launch serves a decode step (one row per sequence) and a prompt portion of any length; the
 // arithmetic per token does not depend on how the rows were cut into steps.
 #include "rows_f32.h"
@@ -22,8 +21,6 @@
 namespace {
 using namespace rows;
 
-constexpr int VB = 16;   // value columns per workgroup
-constexpr int DP = 16;   // lanes per column
 
 template <typename AT>
 __global__ __launch_bounds__(NT) void mlstm_gates_kernel(float* __restrict__ gates, const AT* __restrict__ h,
@@ -96,182 +93,232 @@ struct ScanArgs {
   int vec;                 // q / k rows can be read in aligned 16-byte pieces
 };
 
-// The scalar part of the recurrence, once per (sequence, head) instead of in every workgroup of the state
-// update: from the running maximum in the sequence's slot (0 for a fresh sequence) the factors of every row,
-//   dec[t, h] = (exp(f + m_prev - m_new), exp(i - m_new), exp(-m_new)),
-// and the new maximum back into the slot.  One thread per head; rows are read eight at a time.
+// The scalar chain, once per (sequence, head) in a launch of its own.  m_t = max(f_t + m_(t-1), i_t) is a
+// recurrence in the (max, +) algebra, whose steps compose associatively ((a, b) then (c, d) is (a + c,
+// max(b + c, d))), so a wave scans 64 rows at a time with shuffles and every lane then forms its own row's
+//   dec[t, h] = (exp(f + m_prev - m), exp(i - m), exp(-m))
+// in parallel; the maximum goes from / to the sequence's slot (0 for a fresh sequence).
 __global__ __launch_bounds__(64) void mlstm_decay_kernel(float* __restrict__ dec, const float* __restrict__ gates,
                                                          float* __restrict__ st_m, ScanArgs a) {
-  const int seq = blockIdx.x, h = blockIdx.y * 64 + threadIdx.x;
+  const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int slot = a.seq_slots[seq];
-  if (slot < 0 || h >= a.H) return;
+  if (slot < 0) return;
   const int r0 = a.q_starts ? a.q_starts[seq] : seq, r1 = a.q_starts ? a.q_starts[seq + 1] : seq + 1;
   if (r1 <= r0) return;
   const int H = a.H;
-  float m = a.positions[r0] == 0 ? 0.f : st_m[(size_t)slot * H + h];
-  for (int t0 = r0; t0 < r1; t0 += 8) {
-    float ig[8], fg[8];
+  float m = a.positions[r0] == 0 ? 0.f : st_m[(size_t)slot * H + h];   // the maximum before the block of 64 rows
+  for (int t0 = r0; t0 < r1; t0 += 64) {
+    const int t = t0 + lane;
+    const bool ok = t < r1;
+    const float ig = ok ? gates[(size_t)t * 2 * H + h] : -INFINITY;   // a row past the end is the identity step (0, -inf)
+    const float fg = ok ? gates[(size_t)t * 2 * H + H + h] : 0.f;
+    float ca = fg, cb = ig;   // the composed step of rows t0 .. t: m -> max(m + ca, cb)
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int t = min(t0 + u, r1 - 1);
-      ig[u] = gates[(size_t)t * 2 * H + h];
-      fg[u] = gates[(size_t)t * 2 * H + H + h];
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      if (t0 + u < r1) {
-        const float mn = fmaxf(fg[u] + m, ig[u]);
-        float* d = dec + ((size_t)(t0 + u) * H + h) * 3;
-        d[0] = expf(fg[u] + m - mn);
-        d[1] = expf(ig[u] - mn);
-        d[2] = expf(-mn);
-        m = mn;
+    for (int off = 1; off < 64; off <<= 1) {
+      const float pa = __shfl_up(ca, off, 64), pb = __shfl_up(cb, off, 64);
+      if (lane >= off) {
+        cb = fmaxf(pb + ca, cb);
+        ca = pa + ca;
       }
     }
+    const float mt = fmaxf(m + ca, cb);
+    float mp = __shfl_up(mt, 1, 64);
+    if (lane == 0) mp = m;
+    if (ok) {
+      float* d = dec + ((size_t)t * H + h) * 3;
+      d[0] = expf(fg + mp - mt);
+      d[1] = expf(ig - mt);
+      d[2] = expf(-mt);
+    }
+    m = __shfl(mt, 63, 64);
   }
-  st_m[(size_t)slot * H + h] = m;
+  if (lane == 0) st_m[(size_t)slot * H + h] = m;
 }
 
-// state layout: S [slots, H, Dv, D] (a column's D entries are contiguous), n [slots, H, D], m [slots, H]
-template <typename AT, int RPT>
-__global__ __launch_bounds__(NT) void mlstm_scan_kernel(float* __restrict__ out, const AT* __restrict__ proj,
-                                                        const float* __restrict__ dec, float* __restrict__ st_S,
-                                                        float* __restrict__ st_n, ScanArgs a, int TB) {
+// rows t0 .. t0 + nt of head h: q (scaled) and k as fp32 into LDS tiles [nt][Dp] (pad entries d >= D are not written)
+template <typename AT>
+KA_DEV void stage_qk(float* qs, float* ks, int Dp, const AT* __restrict__ proj, const ScanArgs& a, int h, int t0, int nt) {
+  const int D = a.D;
+  if (a.vec) {   // 16-byte pieces, all requested before any is unpacked
+    constexpr int CE = 16 / (int)sizeof(AT), MAXIT = 8;
+    const int cpr = D / CE, total = nt * cpr;
+    uint4 rq[MAXIT], rk[MAXIT];
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) {
+      const int idx = threadIdx.x + it * NT;
+      if (idx < total) {
+        const AT* row = proj + (size_t)(t0 + idx / cpr) * a.ps + h * D + (idx % cpr) * CE;
+        rq[it] = *reinterpret_cast<const uint4*>(row + a.q_off);
+        rk[it] = *reinterpret_cast<const uint4*>(row + a.k_off);
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) {
+      const int idx = threadIdx.x + it * NT;
+      if (idx < total) {
+        float* qd = qs + (idx / cpr) * Dp + (idx % cpr) * CE;
+        float* kd = ks + (idx / cpr) * Dp + (idx % cpr) * CE;
+        const uint32_t wq[4] = {rq[it].x, rq[it].y, rq[it].z, rq[it].w}, wk[4] = {rk[it].x, rk[it].y, rk[it].z, rk[it].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if constexpr (sizeof(AT) == 2) {
+            qd[2 * i] = lo_f(wq[i]) * a.qscale;
+            qd[2 * i + 1] = hi_f(wq[i]) * a.qscale;
+            kd[2 * i] = lo_f(wk[i]);
+            kd[2 * i + 1] = hi_f(wk[i]);
+          } else {
+            qd[i] = __uint_as_float(wq[i]) * a.qscale;
+            kd[i] = __uint_as_float(wk[i]);
+          }
+        }
+      }
+    }
+  } else {
+    for (int idx = threadIdx.x; idx < nt * D; idx += NT) {
+      const int tt = idx / D, d = idx % D;
+      const AT* row = proj + (size_t)(t0 + tt) * a.ps + h * D + d;
+      qs[tt * Dp + d] = ldf(row + a.q_off) * a.qscale;
+      ks[tt * Dp + d] = ldf(row + a.k_off);
+    }
+  }
+}
+
+// The state update and read-out.  S [slots, H, Dv, D] (a column's D entries contiguous), n [slots, H, D].
+// The normaliser n obeys the same update as a column of S whose value is 1, and n . q is that column's
+// read-out: the columns of a head are numbered c = 0 .. Dv with c = 0 the normaliser and c >= 1 the value column
+// c - 1.  A column is held by DPL adjacent lanes, each with RPT consecutive entries in registers (the q and k
+// rows come from LDS as broadcast 16-byte pieces); a workgroup takes (sequence, head, 256 / DPL columns).  The
+// numerators go to `out`, the denominators max(|n . q|, exp(-m)) + 1e-6 to `den` [T, H]; the division is the
+// first step of the head norm that follows.
+template <typename AT, int RPT, int DPL>
+__global__ __launch_bounds__(NT) void mlstm_scan_kernel(float* __restrict__ out, float* __restrict__ den,
+                                                        const AT* __restrict__ proj, const float* __restrict__ dec,
+                                                        float* __restrict__ st_S, float* __restrict__ st_n, ScanArgs a,
+                                                        int TB) {
   extern __shared__ float lds[];
-  constexpr int Dp = DP * RPT;          // D padded
+  constexpr int Dp = DPL * RPT, CW = NT / DPL;   // D padded; columns per workgroup
   float* qs = lds;                      // [TB][Dp]
   float* ks = qs + TB * Dp;             // [TB][Dp]
-  float* vs = ks + TB * Dp;             // [TB][VB]
-  float* df = vs + TB * VB;             // [TB][3] the row's factors (forget, input, exp(-maximum))
-  const int seq = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * VB;
+  float* vs = ks + TB * Dp;             // [TB][CW]
+  float* df = vs + TB * CW;             // [TB][3] the row's factors (forget, input, exp(-maximum))
+  const int seq = blockIdx.x, h = blockIdx.y;
   const int slot = a.seq_slots[seq];
   if (slot < 0) return;
   const int r0 = a.q_starts ? a.q_starts[seq] : seq, r1 = a.q_starts ? a.q_starts[seq + 1] : seq + 1;
   if (r1 <= r0) return;
   const int H = a.H, D = a.D, Dv = a.Dv;
-  const int col = threadIdx.x / DP, dp = threadIdx.x % DP;
-  const int v = v0 + col;
-  const bool vok = v < Dv;
-  float S[RPT], n[RPT];
-  float* Sp = st_S + (((size_t)slot * H + h) * Dv + (vok ? v : 0)) * D;
-  float* np = st_n + ((size_t)slot * H + h) * D;
+  const int col = threadIdx.x / DPL, dp = threadIdx.x % DPL;
+  const int c = blockIdx.z * CW + col;            // 0: the normaliser, else value column c - 1
+  const bool cok = c <= Dv;
+  float* Sp = c == 0 ? st_n + ((size_t)slot * H + h) * D : st_S + (((size_t)slot * H + h) * Dv + (cok ? c - 1 : 0)) * D;
   const bool fresh = a.positions[r0] == 0;
+  float S[RPT];
+  const bool whole = cok && (dp + 1) * RPT <= D && (D & 3) == 0;   // this lane's entries in aligned 16-byte pieces
 #pragma unroll
-  for (int r = 0; r < RPT; ++r) {
-    const int d = dp + DP * r;
-    const bool ok = !fresh && d < D;
-    S[r] = ok && vok ? Sp[d] : 0.f;
-    n[r] = ok ? np[d] : 0.f;
+  for (int u = 0; u < RPT / 4; ++u) {
+    f32x4 x = {0.f, 0.f, 0.f, 0.f};
+    if (!fresh) {
+      if (whole) {
+        x = *reinterpret_cast<const f32x4*>(Sp + dp * RPT + 4 * u);
+      } else if (cok) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (dp * RPT + 4 * u + i < D) x[i] = Sp[dp * RPT + 4 * u + i];
+      }
+    }
+    S[4 * u] = x[0];
+    S[4 * u + 1] = x[1];
+    S[4 * u + 2] = x[2];
+    S[4 * u + 3] = x[3];
   }
-  if (a.vec)
+  if (Dp != D)
     for (int idx = threadIdx.x; idx < 2 * TB * Dp; idx += NT) qs[idx] = 0.f;   // q and k tiles, pad entries included
+  const int c0 = blockIdx.z * CW;
   for (int t0 = r0; t0 < r1; t0 += TB) {
     const int nt = min(TB, r1 - t0);
     __syncthreads();
-    if (a.vec) {
-      // 16-byte pieces of the q and k rows, all requested before any is unpacked (the pad entries d >= D stay 0)
-      constexpr int CE = 16 / (int)sizeof(AT), MAXIT = 8;
-      const int cpr = D / CE, total = nt * cpr;
-      uint4 rq[MAXIT], rk[MAXIT];
-#pragma unroll
-      for (int it = 0; it < MAXIT; ++it) {
-        const int idx = threadIdx.x + it * NT;
-        if (idx < total) {
-          const AT* row = proj + (size_t)(t0 + idx / cpr) * a.ps + h * D + (idx % cpr) * CE;
-          rq[it] = *reinterpret_cast<const uint4*>(row + a.q_off);
-          rk[it] = *reinterpret_cast<const uint4*>(row + a.k_off);
-        }
-      }
-#pragma unroll
-      for (int it = 0; it < MAXIT; ++it) {
-        const int idx = threadIdx.x + it * NT;
-        if (idx < total) {
-          float* qd = qs + (idx / cpr) * Dp + (idx % cpr) * CE;
-          float* kd = ks + (idx / cpr) * Dp + (idx % cpr) * CE;
-          const uint32_t wq[4] = {rq[it].x, rq[it].y, rq[it].z, rq[it].w}, wk[4] = {rk[it].x, rk[it].y, rk[it].z, rk[it].w};
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            if constexpr (sizeof(AT) == 2) {
-              qd[2 * i] = lo_f(wq[i]) * a.qscale;
-              qd[2 * i + 1] = hi_f(wq[i]) * a.qscale;
-              kd[2 * i] = lo_f(wk[i]);
-              kd[2 * i + 1] = hi_f(wk[i]);
-            } else {
-              qd[i] = __uint_as_float(wq[i]) * a.qscale;
-              kd[i] = __uint_as_float(wk[i]);
-            }
-          }
-        }
-      }
-    } else {
-      for (int idx = threadIdx.x; idx < nt * Dp; idx += NT) {
-        const int tt = idx / Dp, d = idx % Dp;
-        const AT* row = proj + (size_t)(t0 + tt) * a.ps;
-        qs[idx] = d < D ? ldf(row + a.q_off + h * D + d) * a.qscale : 0.f;
-        ks[idx] = d < D ? ldf(row + a.k_off + h * D + d) : 0.f;
-      }
-    }
-    for (int idx = threadIdx.x; idx < nt * VB; idx += NT) {
-      const int tt = idx / VB, c = idx % VB;
-      vs[idx] = v0 + c < Dv ? ldf(proj + (size_t)(t0 + tt) * a.ps + a.v_off + h * Dv + v0 + c) : 0.f;
+    stage_qk(qs, ks, Dp, proj, a, h, t0, nt);
+    for (int idx = threadIdx.x; idx < nt * CW; idx += NT) {
+      const int tt = idx / CW, cc = c0 + idx % CW;
+      vs[idx] = cc == 0 ? 1.f : (cc <= Dv ? ldf(proj + (size_t)(t0 + tt) * a.ps + a.v_off + h * Dv + cc - 1) : 0.f);
     }
     for (int idx = threadIdx.x; idx < nt * 3; idx += NT) df[idx] = dec[((size_t)(t0 + idx / 3) * H + h) * 3 + idx % 3];
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
-      const float fa = df[tt * 3], ia = df[tt * 3 + 1];
-      const float vv = vs[tt * VB + col] * ia;
-      float pq = 0.f, pn = 0.f;
+      const float fa = df[tt * 3];
+      const float vv = vs[tt * CW + col] * df[tt * 3 + 1];
+      const f32x4* k4 = reinterpret_cast<const f32x4*>(ks + tt * Dp + dp * RPT);
+      const f32x4* q4 = reinterpret_cast<const f32x4*>(qs + tt * Dp + dp * RPT);
+      float p0 = 0.f, p1 = 0.f;
 #pragma unroll
-      for (int r = 0; r < RPT; ++r) {
-        const float kd = ks[tt * Dp + dp + DP * r], qd = qs[tt * Dp + dp + DP * r];
-        S[r] = fa * S[r] + kd * vv;
-        n[r] = fa * n[r] + ia * kd;
-        pq += S[r] * qd;
-        pn += n[r] * qd;
+      for (int u = 0; u < RPT / 4; ++u) {
+        const f32x4 kc = k4[u], qc = q4[u];
+        S[4 * u] = fa * S[4 * u] + kc[0] * vv;
+        S[4 * u + 1] = fa * S[4 * u + 1] + kc[1] * vv;
+        S[4 * u + 2] = fa * S[4 * u + 2] + kc[2] * vv;
+        S[4 * u + 3] = fa * S[4 * u + 3] + kc[3] * vv;
+        p0 += S[4 * u] * qc[0] + S[4 * u + 2] * qc[2];
+        p1 += S[4 * u + 1] * qc[1] + S[4 * u + 3] * qc[3];
       }
-      pq = row16_sum(pq);
-      pn = row16_sum(pn);
-      if (dp == 0 && vok) out[((size_t)(t0 + tt) * H + h) * Dv + v] = pq / (fmaxf(fabsf(pn), df[tt * 3 + 2]) + 1e-6f);
+      float pq = p0 + p1;
+      if constexpr (DPL == 4) {
+        pq += dpp_f<0xB1>(pq);
+        pq += dpp_f<0x4E>(pq);
+      } else {
+        pq = row16_sum(pq);
+      }
+      if (dp == 0 && cok) {
+        if (c == 0) den[(size_t)(t0 + tt) * H + h] = fmaxf(fabsf(pq), df[tt * 3 + 2]) + 1e-6f;
+        else out[((size_t)(t0 + tt) * H + h) * Dv + c - 1] = pq;
+      }
     }
   }
+  if (whole) {
 #pragma unroll
-  for (int r = 0; r < RPT; ++r) {
-    const int d = dp + DP * r;
-    if (d < D) {
-      if (vok) Sp[d] = S[r];
-      if (blockIdx.z == 0 && col == 0) np[d] = n[r];
+    for (int u = 0; u < RPT / 4; ++u)
+      *reinterpret_cast<f32x4*>(Sp + dp * RPT + 4 * u) = f32x4{S[4 * u], S[4 * u + 1], S[4 * u + 2], S[4 * u + 3]};
+  } else if (cok) {
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) {
+      const int d = dp * RPT + r;
+      if (d < D) Sp[d] = S[r];
     }
   }
 }
 
-template <typename AT, int RPT>
-int launch_scan(float* out, const AT* proj, const float* dec, float* S, float* n, const ScanArgs& a, int num_seqs,
+template <typename AT, int RPT, int DPL>
+int launch_scan(float* out, float* den, const AT* proj, const float* dec, float* S, float* n, ScanArgs a, int num_seqs,
                 hipStream_t st) {
-  // rows staged per tile: as many as 32 KB of q and k allow, 16 .. 64
-  int TB = 4096 / (DP * RPT);
+  constexpr int Dp = RPT * DPL, CW = NT / DPL;
+  int TB = 4096 / Dp;   // rows staged per tile: as many as 32 KB of q and k allow, 16 .. 64
   TB = TB < 16 ? 16 : (TB > 64 ? 64 : TB);
-  const size_t lds = (size_t)(2 * TB * DP * RPT + TB * VB + 3 * TB) * sizeof(float);
+  const int ce = 16 / (int)sizeof(AT);
+  a.vec = a.D % ce == 0 && a.ps % ce == 0 && a.q_off % ce == 0 && a.k_off % ce == 0 && ((uintptr_t)proj & 15) == 0 &&
+          TB * (a.D / ce) <= 8 * NT;
+  const size_t lds = (size_t)(2 * TB * Dp + TB * CW + 3 * TB) * sizeof(float);
   if (lds > 48 * 1024) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mlstm_scan_kernel<AT, RPT>),
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mlstm_scan_kernel<AT, RPT, DPL>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  dim3 grid(num_seqs, a.H, (a.Dv + VB - 1) / VB);
-  mlstm_scan_kernel<AT, RPT><<<grid, NT, lds, st>>>(out, proj, dec, S, n, a, TB);
+  dim3 grid(num_seqs, a.H, (a.Dv + 1 + CW - 1) / CW);
+  mlstm_scan_kernel<AT, RPT, DPL><<<grid, NT, lds, st>>>(out, den, proj, dec, S, n, a, TB);
   KA_CHECK_LAUNCH();
 }
 
 template <typename AT>
-int dispatch_scan(float* out, const AT* proj, const float* dec, float* S, float* n, const ScanArgs& a, int num_seqs,
-                  hipStream_t st) {
-  const int need = (a.D + DP - 1) / DP;
-  if (need <= 1) return launch_scan<AT, 1>(out, proj, dec, S, n, a, num_seqs, st);
-  if (need <= 2) return launch_scan<AT, 2>(out, proj, dec, S, n, a, num_seqs, st);
-  if (need <= 4) return launch_scan<AT, 4>(out, proj, dec, S, n, a, num_seqs, st);
-  if (need <= 8) return launch_scan<AT, 8>(out, proj, dec, S, n, a, num_seqs, st);
-  if (need <= 16) return launch_scan<AT, 16>(out, proj, dec, S, n, a, num_seqs, st);
-  if (need <= 32) return launch_scan<AT, 32>(out, proj, dec, S, n, a, num_seqs, st);
-  return (int)hipErrorInvalidValue;
+int dispatch_scan(float* out, float* den, const AT* proj, const float* gates, float* dec, float* S, float* n, float* m,
+                  const ScanArgs& a, int num_seqs, hipStream_t st) {
+  mlstm_decay_kernel<<<dim3(num_seqs, a.H), 64, 0, st>>>(dec, gates, m, a);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return (int)e;
+  const int D = a.D;
+  if (D <= 16) return launch_scan<AT, 4, 4>(out, den, proj, dec, S, n, a, num_seqs, st);
+  if (D <= 32) return launch_scan<AT, 8, 4>(out, den, proj, dec, S, n, a, num_seqs, st);
+  if (D <= 64) return launch_scan<AT, 16, 4>(out, den, proj, dec, S, n, a, num_seqs, st);
+  if (D <= 128) return launch_scan<AT, 32, 4>(out, den, proj, dec, S, n, a, num_seqs, st);
+  if (D <= 256) return launch_scan<AT, 64, 4>(out, den, proj, dec, S, n, a, num_seqs, st);
+  return launch_scan<AT, 32, 16>(out, den, proj, dec, S, n, a, num_seqs, st);
 }
 
 }  // namespace
@@ -284,24 +331,17 @@ extern "C" int ka_mlstm_gates(float* gates, const void* h, const float* w, const
   KA_CHECK_LAUNCH();
 }
 
-// dec: scratch [T, H, 3] fp32 (the rows' factors, written by the first launch and read by the second)
-extern "C" int ka_mlstm_scan(float* out, const void* proj, int ps, int q_off, int k_off, int v_off, const float* gates,
-                             float* dec, float* st_S, float* st_n, float* st_m, const int* seq_slots, const int* q_starts,
-                             int num_seqs, const int* positions, int H, int D, int Dv, float qscale, int f32,
-                             hipStream_t st) {
+// out [T, H * Dv]: the numerators; den [T, H]: the denominators; dec: scratch [T, H, 3] fp32 (the rows' factors,
+// written by the first launch and read by the second)
+extern "C" int ka_mlstm_scan(float* out, float* den, const void* proj, int ps, int q_off, int k_off, int v_off,
+                             const float* gates, float* dec, float* st_S, float* st_n, float* st_m, const int* seq_slots,
+                             const int* q_starts, int num_seqs, const int* positions, int H, int D, int Dv, float qscale,
+                             int f32, hipStream_t st) {
   if (num_seqs <= 0) return 0;
-  if (H <= 0 || D <= 0 || Dv <= 0 || H > 65535) return (int)hipErrorInvalidValue;
-  const int ce = f32 ? 4 : 8;
-  const int need = (D + DP - 1) / DP;
-  const int rpt = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : need <= 8 ? 8 : need <= 16 ? 16 : 32;
-  int tb = 4096 / (DP * rpt);
-  tb = tb < 16 ? 16 : (tb > 64 ? 64 : tb);
-  const int vec = D % ce == 0 && ps % ce == 0 && q_off % ce == 0 && k_off % ce == 0 &&
-                  ((uintptr_t)proj & 15) == 0 && tb * (D / ce) <= 8 * NT;
-  ScanArgs a{q_starts, seq_slots, positions, ps, q_off, k_off, v_off, H, D, Dv, qscale, vec};
-  mlstm_decay_kernel<<<dim3(num_seqs, (H + 63) / 64), 64, 0, st>>>(dec, gates, st_m, a);
-  if (f32) return dispatch_scan<float>(out, (const float*)proj, dec, st_S, st_n, a, num_seqs, st);
-  return dispatch_scan<bf16_t>(out, (const bf16_t*)proj, dec, st_S, st_n, a, num_seqs, st);
+  if (H <= 0 || D <= 0 || D > 512 || Dv <= 0 || H > 65535) return (int)hipErrorInvalidValue;
+  ScanArgs a{q_starts, seq_slots, positions, ps, q_off, k_off, v_off, H, D, Dv, qscale, 0};
+  if (f32) return dispatch_scan<float>(out, den, (const float*)proj, gates, dec, st_S, st_n, st_m, a, num_seqs, st);
+  return dispatch_scan<bf16_t>(out, den, (const bf16_t*)proj, gates, dec, st_S, st_n, st_m, a, num_seqs, st);
 }
 
 // bf16 activations with a bf16 copy of the gate weights [2H, width]; width a multiple of 128, 2H <= 128

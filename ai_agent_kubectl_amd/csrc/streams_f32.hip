@@ -9,7 +9,7 @@
 //
 // S = 1 with w_in = mix = out = 1 is the plain pre-norm residual.  Also here: the embedding gather into
 // the S copies with a scale, relu(z)^2, silu(gate) * up, and the per-head RMS division with an output
-// gate that closes an mLSTM (out = o / rms_head(o) * w * sigmoid(g)).
+// gate that closes an mLSTM (o <- o / den; out = o / rms_head(o) * w * sigmoid(g)).
 #include "rows_f32.h"
 
 namespace {
@@ -127,16 +127,22 @@ __global__ __launch_bounds__(NT) void silu_mul_rows_kernel(AT* __restrict__ out,
 }
 
 // one wave per head: o [T, H * Dv] fp32 -> out in AT; the gate columns sit in `proj` rows of stride ps at g_off
+// den [T, H] (optional): the head's entries are first divided by den[t, h]
 template <typename AT>
 __global__ __launch_bounds__(NT) void headnorm_gate_kernel(AT* __restrict__ out, const float* __restrict__ o,
-                                                           const AT* __restrict__ proj, int ps, int g_off,
-                                                           const float* __restrict__ w, int H, int Dv, float eps) {
+                                                           const float* __restrict__ den, const AT* __restrict__ proj,
+                                                           int ps, int g_off, const float* __restrict__ w, int H, int Dv,
+                                                           float eps) {
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int h = wave; h < H; h += NW) {
     const float* oh = o + ((size_t)t * H + h) * Dv;
+    const float rd = den != nullptr ? 1.0f / den[(size_t)t * H + h] : 1.0f;
     float ss = 0.f;
-    for (int i = lane; i < Dv; i += 64) ss += oh[i] * oh[i];
-    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)Dv + eps);
+    for (int i = lane; i < Dv; i += 64) {
+      const float v = oh[i] * rd;
+      ss += v * v;
+    }
+    const float inv = rd / sqrtf(wave_sum(ss) / (float)Dv + eps);
     for (int i = lane; i < Dv; i += 64) {
       const float g = ldf(proj + (size_t)t * ps + g_off + h * Dv + i);
       stf(out + ((size_t)t * H + h) * Dv + i, oh[i] * inv * w[h * Dv + i] / (1.f + expf(-g)));
@@ -196,10 +202,10 @@ extern "C" int ka_silu_mul_rows(void* out, const void* gu, int rows_, int ff, in
   KA_CHECK_LAUNCH();
 }
 
-extern "C" int ka_headnorm_gate(void* out, const float* o, const void* proj, int ps, int g_off, const float* w, int T,
-                                int H, int Dv, float eps, int f32, hipStream_t st) {
+extern "C" int ka_headnorm_gate(void* out, const float* o, const float* den, const void* proj, int ps, int g_off,
+                                const float* w, int T, int H, int Dv, float eps, int f32, hipStream_t st) {
   if (T <= 0) return 0;
-  if (f32) headnorm_gate_kernel<float><<<T, NT, 0, st>>>((float*)out, o, (const float*)proj, ps, g_off, w, H, Dv, eps);
-  else headnorm_gate_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)out, o, (const bf16_t*)proj, ps, g_off, w, H, Dv, eps);
+  if (f32) headnorm_gate_kernel<float><<<T, NT, 0, st>>>((float*)out, o, den, (const float*)proj, ps, g_off, w, H, Dv, eps);
+  else headnorm_gate_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)out, o, den, (const bf16_t*)proj, ps, g_off, w, H, Dv, eps);
   KA_CHECK_LAUNCH();
 }

@@ -7,8 +7,9 @@ and updates every copy (hyper-connections; S = 1 with unit weights is the plain 
 
 Mixers (activations in the engine dtype, bf16 or fp32; what is marked fp32 is fp32 in both):
   mLSTM            [q | k | v | g] = h @ w_proj^T (one vendor GEMM); log gates from h in fp32 (mlstm_gates);
-                   the recurrence over the step's rows from / into the sequence's state slot, fp32 (mlstm_scan);
-                   per-head RMS division, weight, sigmoid(g) gate (headnorm_gate); output GEMM.
+                   the recurrence over the step's rows from / into the sequence's state slot, fp32 (mlstm_scan:
+                   numerators and denominators); division, per-head RMS division, weight, sigmoid(g) gate
+                   (headnorm_gate); output GEMM.
   latent attention [c_q | c | k_r] = h @ w_dn^T (one GEMM); RMS norm of c_q, RMS norm of c and rotary on k_r
                    appended to the paged cache (latent_prep); q = c_q @ w_uq^T; rotary on q's rotated part
                    and the unrotated parts carried into the latent space by a batched GEMM with w_uk
@@ -107,11 +108,11 @@ class KafilornModel:
         proj = F.linear(h, L["w_proj"])                                # [T, q | k | v | g]
         gates = mixers.mlstm_gates(h, L["w_if"], L["b_if"], m.gate_cap, L.get("w_if_lp"))
         S, n, mx = self.state[li]
-        o = mixers.mlstm_scan(proj, 0, HD, 2 * HD, gates, S, n, mx, meta.state_slots,
-                              None if meta.is_decode else meta.q_starts, meta.positions, m.heads, m.dim, m.vdim,
-                              m.dim ** -0.5)
+        o, den = mixers.mlstm_scan(proj, 0, HD, 2 * HD, gates, S, n, mx, meta.state_slots,
+                                   None if meta.is_decode else meta.q_starts, meta.positions, m.heads, m.dim, m.vdim,
+                                   m.dim ** -0.5)
         return F.linear(mixers.headnorm_gate(o, proj, 2 * HD + HV, L["hnorm"], m.heads, m.vdim, self.cfg.norm_eps,
-                                             self.dtype), L["wo"])
+                                             self.dtype, den), L["wo"])
 
     def _latent_attention(self, h, L, m, cache, meta: AttnMeta):
         T = h.shape[0]

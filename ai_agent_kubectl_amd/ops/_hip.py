@@ -120,10 +120,10 @@ _MIX_SIGS = {
     "ka_stream_update": [P, P, P, P, P, P, P, I, I, I, F, I, I, P],
     "ka_relu_sq": [P, P, ctypes.c_long, I, P],
     "ka_silu_mul_rows": [P, P, I, I, I, P],
-    "ka_headnorm_gate": [P, P, P, I, I, P, I, I, I, F, I, P],
+    "ka_headnorm_gate": [P, P, P, P, I, I, P, I, I, I, F, I, P],
     "ka_mlstm_gates": [P, P, P, P, I, I, I, F, I, P],
     "ka_mlstm_gates_mfma": [P, P, P, P, I, I, I, F, P],
-    "ka_mlstm_scan": [P, P, I, I, I, I, P, P, P, P, P, P, P, I, P, I, I, I, F, I, P],
+    "ka_mlstm_scan": [P, P, P, I, I, I, I, P, P, P, P, P, P, P, I, P, I, I, I, F, I, P],
     "ka_latent_prep": [P, P, I, I, I, I, I, P, P, P, P, P, P, I, F, I, P],
     "ka_rope_split_q": [P, P, P, P, P, I, I, I, I, I, I, P],
     "ka_window_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, P],

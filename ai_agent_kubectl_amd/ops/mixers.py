@@ -270,7 +270,8 @@ def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gates: to
                positions: torch.Tensor, H: int, D: int, Dv: int, qscale: float) -> torch.Tensor:
     """The mLSTM recurrence over each sequence's rows, from / into the state of its slot (st_S [slots, H, Dv, D],
     st_n [slots, H, D], st_m [slots, H], fp32); a sequence whose first row is at position 0 starts from zero.
-    q_starts None: row t is sequence t.  -> [T, H * Dv] fp32 (numerator / denominator, before the head norm)."""
+    q_starts None: row t is sequence t.  -> (numerators S^T q [T, H * Dv], denominators max(|n . q|, exp(-m)) + 1e-6
+    [T, H]), fp32; `headnorm_gate` divides."""
     if _ref(proj):
         S = st_S.transpose(-1, -2)
         return ref.mlstm_scan(proj, q_off, k_off, v_off, gates, S, st_n, st_m, seq_slots, q_starts, positions, H, D, Dv,
@@ -286,25 +287,28 @@ def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gates: to
     assert (q_starts is None and nseq <= T) or (q_starts is not None and q_starts.dtype == torch.int32
                                                  and q_starts.shape[0] == nseq + 1)
     out = torch.zeros((T, H * Dv), dtype=torch.float32, device=proj.device)
+    den = torch.ones((T, H), dtype=torch.float32, device=proj.device)
     dec = torch.empty((T, H, 3), dtype=torch.float32, device=proj.device)   # per row: forget factor, input factor, exp(-max)
-    check(lib.ka_mlstm_scan(_p(out), _p(proj), P, q_off, k_off, v_off, _p(gates), _p(dec), _p(st_S), _p(st_n), _p(st_m),
-                            _p(seq_slots), _p(q_starts), nseq, _p(positions), H, D, Dv, float(qscale), _f32(proj),
+    check(lib.ka_mlstm_scan(_p(out), _p(den), _p(proj), P, q_off, k_off, v_off, _p(gates), _p(dec), _p(st_S), _p(st_n),
+                            _p(st_m), _p(seq_slots), _p(q_starts), nseq, _p(positions), H, D, Dv, float(qscale), _f32(proj),
                             _stream()), "mlstm_scan")
-    return out
+    return out, den
 
 
 def headnorm_gate(o: torch.Tensor, proj: torch.Tensor, g_off: int, w: torch.Tensor, H: int, Dv: int, eps: float,
-                  out_dtype) -> torch.Tensor:
-    """o [T, H * Dv] fp32: each head divided by its root mean square, times w, times sigmoid(proj[:, g_off:...])."""
+                  out_dtype, den: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """o [T, H * Dv] fp32 (each head first divided by den [T, H], if given): each head divided by its root mean
+    square, times w, times sigmoid(proj[:, g_off:...])."""
     if _ref(o):
-        return ref.headnorm_gate(o, proj, g_off, w, H, Dv, eps, out_dtype)
+        return ref.headnorm_gate(o, proj, g_off, w, H, Dv, eps, out_dtype, den)
     lib = require_mixers()
     T = o.shape[0]
     assert o.dtype == torch.float32 and o.is_contiguous() and proj.is_contiguous() and proj.dtype == out_dtype
     assert g_off + H * Dv <= proj.shape[1] and w.dtype == torch.float32 and w.numel() == H * Dv
+    assert den is None or (den.dtype == torch.float32 and den.shape == (T, H) and den.is_contiguous())
     out = torch.empty((T, H * Dv), dtype=out_dtype, device=o.device)
-    check(lib.ka_headnorm_gate(_p(out), _p(o), _p(proj), proj.shape[1], g_off, _p(w), T, H, Dv, float(eps), _f32(out),
-                               _stream()), "headnorm_gate")
+    check(lib.ka_headnorm_gate(_p(out), _p(o), _p(den), _p(proj), proj.shape[1], g_off, _p(w), T, H, Dv, float(eps),
+                               _f32(out), _stream()), "headnorm_gate")
     return out
 
 

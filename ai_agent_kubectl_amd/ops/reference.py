@@ -291,9 +291,10 @@ def mlstm_scan(proj, q_off: int, k_off: int, v_off: int, gates, st_S, st_n, st_m
                H: int, D: int, Dv: int, qscale: float) -> torch.Tensor:
     """The recurrence over each sequence's rows of this step, from the state in its slot (zero when the row's
     position is 0) and back into it.  proj rows hold q [H, D], k [H, D], v [H, Dv] at the given column offsets.
-    -> num / den per head [T, H * Dv] fp32 (before the head norm)."""
+    -> (numerators S^T q [T, H * Dv], denominators max(|n . q|, exp(-m)) + 1e-6 [T, H]), fp32."""
     T = proj.shape[0]
     out = torch.zeros((T, H * Dv), dtype=torch.float32, device=proj.device)
+    dens = torch.ones((T, H), dtype=torch.float32, device=proj.device)
     slots, pos = seq_slots.tolist(), positions.tolist()
     for i, a, b in _seq_of(T, q_starts):
         sl = slots[i]
@@ -313,16 +314,19 @@ def mlstm_scan(proj, q_off: int, k_off: int, v_off: int, gates, st_S, st_n, st_m
             S = fa[:, None, None] * S + ia[:, None, None] * (k[:, :, None] * v[:, None, :])
             n = fa[:, None] * n + ia[:, None] * k
             m = m_new
-            den = torch.maximum((n * q).sum(-1).abs(), torch.exp(-m)) + 1e-6
-            out[t] = (torch.einsum("hdv,hd->hv", S, q) / den[:, None]).reshape(-1)
+            dens[t] = torch.maximum((n * q).sum(-1).abs(), torch.exp(-m)) + 1e-6
+            out[t] = torch.einsum("hdv,hd->hv", S, q).reshape(-1)
         st_S[sl], st_n[sl], st_m[sl] = S, n, m
-    return out
+    return out, dens
 
 
-def headnorm_gate(o, proj, g_off: int, w, H: int, Dv: int, eps: float, out_dtype) -> torch.Tensor:
-    """Each head of o divided by its root mean square, times w, times sigmoid(gate columns of proj)."""
+def headnorm_gate(o, proj, g_off: int, w, H: int, Dv: int, eps: float, out_dtype, den=None) -> torch.Tensor:
+    """Each head of o (divided by den [T, H] first, if given) divided by its root mean square, times w, times
+    sigmoid(gate columns of proj)."""
     T = o.shape[0]
     oh = o.view(T, H, Dv)
+    if den is not None:
+        oh = oh / den[:, :, None]
     y = (oh / torch.sqrt((oh * oh).mean(-1, keepdim=True) + eps)).reshape(T, H * Dv) * w.float()
     return (y * torch.sigmoid(proj[:, g_off:g_off + H * Dv].float())).to(out_dtype)
 

@@ -180,9 +180,9 @@ def _mlstm_through_ops(m, P, hs, device, cuts, slot=1, slots=3):
         proj = h @ w_proj.t()
         gates = mixers.mlstm_gates(h, w_if, b_if, float(m.get("gate_cap") or 0.0))
         pos = torch.arange(at, at + c, dtype=torch.int32, device=device)
-        o = mixers.mlstm_scan(proj, 0, H * D, 2 * H * D, gates, *st, torch.tensor([slot], dtype=torch.int32, device=device),
-                              torch.tensor([0, c], dtype=torch.int32, device=device), pos, H, D, Dv, D ** -0.5)
-        y = mixers.headnorm_gate(o, proj, 2 * H * D + H * Dv, f32(P["norm"]), H, Dv, 1e-6, torch.float32)
+        o, den = mixers.mlstm_scan(proj, 0, H * D, 2 * H * D, gates, *st, torch.tensor([slot], dtype=torch.int32, device=device),
+                                   torch.tensor([0, c], dtype=torch.int32, device=device), pos, H, D, Dv, D ** -0.5)
+        y = mixers.headnorm_gate(o, proj, 2 * H * D + H * Dv, f32(P["norm"]), H, Dv, 1e-6, torch.float32, den)
         out.append((y @ f32(P["o"]).t()).cpu())
         at += c
     return torch.cat(out)
