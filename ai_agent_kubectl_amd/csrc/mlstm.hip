@@ -59,7 +59,7 @@ __global__ __launch_bounds__(NT) void mlstm_gates_mfma_kernel(float* __restrict_
     acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const int kper = width / NW, kbeg = wave * kper;
-#pragma unroll 4
+#pragma unroll 8
   for (int k0 = kbeg; k0 < kbeg + kper; k0 += 32) {
     const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(hr + k0));
 #pragma unroll

@@ -34,7 +34,25 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(int* __restrict__ ids, fl
   for (int e = wave; e < E; e += NW) {
     const float* we = wr + (size_t)e * width;
     float s = 0.f;
-    for (int i = lane; i < width; i += 64) s += ldf(hr + i) * we[i];
+    if ((width & 7) == 0) {   // eight entries per lane and trip, 16-byte loads, four trips in flight
+#pragma unroll 4
+      for (int i = 8 * lane; i < width; i += 512) {
+        const f32x4 wa = *reinterpret_cast<const f32x4*>(we + i), wb = *reinterpret_cast<const f32x4*>(we + i + 4);
+        float x[8];
+        if constexpr (sizeof(AT) == 2) {
+          const uint4 hv = *reinterpret_cast<const uint4*>(hr + i);
+          x[0] = lo_f(hv.x); x[1] = hi_f(hv.x); x[2] = lo_f(hv.y); x[3] = hi_f(hv.y);
+          x[4] = lo_f(hv.z); x[5] = hi_f(hv.z); x[6] = lo_f(hv.w); x[7] = hi_f(hv.w);
+        } else {
+          const f32x4 ha = *reinterpret_cast<const f32x4*>(hr + i), hb = *reinterpret_cast<const f32x4*>(hr + i + 4);
+          x[0] = ha[0]; x[1] = ha[1]; x[2] = ha[2]; x[3] = ha[3];
+          x[4] = hb[0]; x[5] = hb[1]; x[6] = hb[2]; x[7] = hb[3];
+        }
+        s += x[0] * wa[0] + x[1] * wa[1] + x[2] * wa[2] + x[3] * wa[3] + x[4] * wb[0] + x[5] * wb[1] + x[6] * wb[2] + x[7] * wb[3];
+      }
+    } else {
+      for (int i = lane; i < width; i += 64) s += ldf(hr + i) * we[i];
+    }
     s = wave_sum(s);
     if (lane == 0) z[e] = s;
   }

@@ -56,6 +56,7 @@ __global__ __launch_bounds__(NT) void stream_norm_kernel(OT* __restrict__ out, c
   float* row = lds;            // [width]
   float* red = lds + width;    // [NW]
   const float* xr = x + (size_t)blockIdx.x * S * width;
+#pragma unroll 4
   for (int i = threadIdx.x; i < width; i += NT) {
     float u = 0.f;
     for (int s = 0; s < S; ++s) u += w_in[s] * xr[(size_t)s * width + i];
@@ -83,6 +84,7 @@ __global__ __launch_bounds__(NT) void stream_update_kernel(float* __restrict__ x
   __syncthreads();
   float* xr = x + (size_t)blockIdx.x * S * width;
   const YT* yr = y + (size_t)blockIdx.x * width;
+#pragma unroll 4
   for (int i = threadIdx.x; i < width; i += NT) {
     float old[MAX_STREAMS];
 #pragma unroll
