@@ -600,7 +600,8 @@ def test_graph_decode_matches_eager(tmp_path, dtype):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("H,R,Dr,window,decode", [(16, 128, 32, 40, False), (4, 64, 0, 0, False), (20, 256, 64, 100, False),
-                                                  (40, 512, 64, 333, False), (16, 128, 32, 40, True), (33, 96, 32, 17, True),
+                                                  (3, 32, 32, 9, False), (6, 48, 16, 50, True),
+                                                  (40, 512, 64, 333, False), (16, 128, 32, 40, True), (33, 160, 32, 17, True),
                                                   (8, 512, 64, 0, True)])
 def test_window_attention_matrix_core_kernel(H, R, Dr, window, decode):
     """bf16 shapes the matrix-core kernel takes (heads below / at / above a 16-head tile and not multiples of it,
