@@ -13,7 +13,7 @@
 // log-sigmoid.  `mlstm_scan`: the recurrence over the rows that each sequence brings to this step, from the
 // state in the sequence's slot and back into it; a row at position 0 starts from the zero state, so a slot
 // needs no clearing between requests.  The scalar chain (running maximum, the rows' factors) runs once per
-// (sequence, head) in a launch of its own, as a parallel scan; the state update follows (below).
+// (sequence, head) in a launch of its own; the state update follows (below).
 // The same launch serves a decode step (one row per sequence) and a prompt portion of any length; the
 // arithmetic per token does not depend on how the rows were cut into steps.
 #include "rows_f32.h"
@@ -93,9 +93,10 @@ struct ScanArgs {
   int vec;                 // q / k rows can be read in aligned 16-byte pieces
 };
 
-// The scalar chain, once per (sequence, head) in a launch of its own.  m_t = max(f_t + m_(t-1), i_t) is a
-// recurrence in the (max, +) algebra, whose steps compose associatively ((a, b) then (c, d) is (a + c,
-// max(b + c, d))), so a wave scans 64 rows at a time with shuffles and every lane then forms its own row's
+// The scalar chain, once per (sequence, head) in a launch of its own: a wave takes 64 rows at a time, every lane
+// loads its row's gates, the chain m_t = max(f_t + m_(t-1), i_t) runs over the 64 rows on lane-broadcast values
+// (two operations a row, the same expression and order as a row-by-row decode, so the factors do not depend on how
+// a prompt was cut), and every lane then forms its own row's
 //   dec[t, h] = (exp(f + m_prev - m), exp(i - m), exp(-m))
 // in parallel; the maximum goes from / to the sequence's slot (0 for a fresh sequence).
 __global__ __launch_bounds__(64) void mlstm_decay_kernel(float* __restrict__ dec, const float* __restrict__ gates,
@@ -106,31 +107,30 @@ __global__ __launch_bounds__(64) void mlstm_decay_kernel(float* __restrict__ dec
   const int r0 = a.q_starts ? a.q_starts[seq] : seq, r1 = a.q_starts ? a.q_starts[seq + 1] : seq + 1;
   if (r1 <= r0) return;
   const int H = a.H;
-  float m = a.positions[r0] == 0 ? 0.f : st_m[(size_t)slot * H + h];   // the maximum before the block of 64 rows
+  float m = a.positions[r0] == 0 ? 0.f : st_m[(size_t)slot * H + h];   // the maximum before the block (the same in every lane)
   for (int t0 = r0; t0 < r1; t0 += 64) {
     const int t = t0 + lane;
     const bool ok = t < r1;
-    const float ig = ok ? gates[(size_t)t * 2 * H + h] : -INFINITY;   // a row past the end is the identity step (0, -inf)
+    const float ig = ok ? gates[(size_t)t * 2 * H + h] : -INFINITY;   // a row past the end leaves the maximum as it is
     const float fg = ok ? gates[(size_t)t * 2 * H + H + h] : 0.f;
-    float ca = fg, cb = ig;   // the composed step of rows t0 .. t: m -> max(m + ca, cb)
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const float pa = __shfl_up(ca, off, 64), pb = __shfl_up(cb, off, 64);
-      if (lane >= off) {
-        cb = fmaxf(pb + ca, cb);
-        ca = pa + ca;
+    float mp = 0.f, mt = 0.f;
+    const int nrow = min(64, r1 - t0);
+    for (int j = 0; j < nrow; ++j) {
+      const float fj = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, fg), j));
+      const float ij = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ig), j));
+      const float prev = m;
+      m = fmaxf(fj + m, ij);
+      if (lane == j) {
+        mp = prev;
+        mt = m;
       }
     }
-    const float mt = fmaxf(m + ca, cb);
-    float mp = __shfl_up(mt, 1, 64);
-    if (lane == 0) mp = m;
     if (ok) {
       float* d = dec + ((size_t)t * H + h) * 3;
       d[0] = expf(fg + mp - mt);
       d[1] = expf(ig - mt);
       d[2] = expf(-mt);
     }
-    m = __shfl(mt, 63, 64);
   }
   if (lane == 0) st_m[(size_t)slot * H + h] = m;
 }
